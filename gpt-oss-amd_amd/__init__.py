@@ -1,0 +1,349 @@
+"""ctypes binding of libmoe_gfx950.so — the gpt-oss MoE expert block for one MI355X (gfx950).
+
+The functions here carry the names and argument order of the reference's host-callable kernels
+(src/hip/gemms/gemm_router.hip:184, src/hip/topk.hip:59, src/hip/softmax.hip:46,
+src/hip/moe.hip:237 and :514, src/hip/vecadd.hip:32) and pass torch device tensors straight
+through to the C ABI declared in include/moe_abi.h.  torch is used for device memory and streams
+only; all arithmetic runs in the HIP library.  There is no CPU fallback: if the library has not
+been built, importing this package raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmoe_gfx950.so")
+
+MOE_WEIGHTS_BF16 = 0
+MOE_WEIGHTS_MXFP4_TILED = 1
+MOE_FLAG_ROUTER_STRICT_ORDER = 1
+MOE_FLAG_FORCE_STREAM = 2
+MOE_FLAG_FORCE_TILED = 4
+
+_c = ctypes
+_vp, _i, _ll, _f, _u, _sz = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float, _c.c_uint, _c.c_size_t
+
+
+class MoeError(RuntimeError):
+    def __init__(self, fn, code):
+        msg = _lib.moe_error_string(code).decode()
+        super().__init__("%s failed: %s (code %d)" % (fn, msg, code))
+        self.code = code
+
+
+class BlockParams(_c.Structure):
+    """moe_block_params of include/moe_abi.h."""
+    _fields_ = [
+        ("struct_bytes", _c.c_uint32),
+        ("n_tokens", _c.c_int32),
+        ("hidden_dim", _c.c_int32),
+        ("intermediate_dim", _c.c_int32),
+        ("n_experts", _c.c_int32),
+        ("experts_per_token", _c.c_int32),
+        ("weight_format", _c.c_int32),
+        ("swiglu_limit", _f),
+        ("alpha", _f),
+        ("t", _vp),
+        ("w_router", _vp),
+        ("b_router", _vp),
+        ("w_mlp1", _vp),
+        ("w_mlp1_scales", _vp),
+        ("b_mlp1", _vp),
+        ("w_mlp2", _vp),
+        ("w_mlp2_scales", _vp),
+        ("b_mlp2", _vp),
+        ("e_agg", _vp),
+        ("topk_i", _vp),
+        ("topk_v", _vp),
+        ("router_score", _vp),
+        ("residual_x", _vp),
+        ("workspace", _vp),
+        ("workspace_bytes", _sz),
+        ("flags", _c.c_uint32),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/moe_abi.h declares
+SIGNATURES = {
+    "moe_abi_version": (_i, []),
+    "moe_error_string": (_c.c_char_p, [_i]),
+    "moe_router_scratch_bytes": (_sz, [_i, _i]),
+    "moe_gemm_router": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
+    "moe_topk": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "moe_softmax": (_i, [_vp, _i, _i, _vp]),
+    "moe_bucket_by_expert": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "moe_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "moe_build_work_queue": (_i, [_vp, _i, _vp, _vp, _vp]),
+    "moe_mlp1_swiglu": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _ll, _ll, _f, _f, _i, _i, _vp]),
+    "moe_mlp2_scatter": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _ll, _ll, _i, _i, _vp]),
+    "moe_mlp1_swiglu_mxfp4": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _ll, _f, _f, _i, _i, _vp]),
+    "moe_mlp2_scatter_mxfp4": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _ll, _i, _i, _vp]),
+    "moe_vecadd_and_zero": (_i, [_vp, _vp, _f, _i, _i, _vp]),
+    "moe_rmsnorm": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "moe_dequant_mxfp4": (_i, [_vp, _vp, _ll, _vp, _vp]),
+    "moe_mxfp4_tiled_bytes": (None, [_i, _i, _c.POINTER(_sz), _c.POINTER(_sz)]),
+    "moe_mxfp4_repack": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
+    "moe_mxfp4_unpack": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
+    "moe_mxfp4_tiled_to_bf16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    "moe_block_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "moe_block_forward": (_i, [_c.POINTER(BlockParams), _vp]),
+    "moe_synth_normal_f32": (_i, [_vp, _ll, _vp, _f, _u, _u, _vp]),
+    "moe_synth_normal_bf16": (_i, [_vp, _ll, _vp, _f, _u, _u, _vp]),
+    "moe_synth_bytes": (_i, [_vp, _ll, _u, _u, _vp]),
+    "moe_synth_range_bytes": (_i, [_vp, _ll, _u, _u, _u, _u, _vp]),
+}
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s is missing: build it with `python gpt-oss-amd_amd/build.py` (hipcc, gfx950). "
+            "There is no CPU fallback for the MoE kernels." % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here = a declared symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+_lib = _load()
+lib = _lib
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    if not t.is_cuda:
+        raise ValueError("expected a device tensor")
+    if not t.is_contiguous():
+        raise ValueError("expected a contiguous tensor")
+    return t.data_ptr()
+
+
+def _stream(stream):
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    return stream.cuda_stream if hasattr(stream, "cuda_stream") else stream
+
+
+def _check(fn, rc):
+    if rc != 0:
+        raise MoeError(fn, rc)
+
+
+# ---- reference-named entry points --------------------------------------------------------------
+def gemm_router(xout, x_batch, w, bias, N, K, M, stream=None, scratch=None):
+    """src/hip/gemms/gemm_router.hip:184 — xout[N,M] = x_batch[N,K] @ w[M,K]^T + bias[M]."""
+    if scratch is None:
+        scratch = torch.empty(_lib.moe_router_scratch_bytes(N, M), dtype=torch.uint8, device=xout.device)
+    _check("moe_gemm_router", _lib.moe_gemm_router(_ptr(xout), _ptr(x_batch), _ptr(w), _ptr(bias), N, K, M,
+                                                   _ptr(scratch), scratch.numel(), _stream(stream)))
+
+
+def topk(topk_values, topk_indices, router_scores, batch_size, num_experts, experts_per_token, stream=None):
+    """src/hip/topk.hip:59."""
+    _check("moe_topk", _lib.moe_topk(_ptr(topk_values), _ptr(topk_indices), _ptr(router_scores), batch_size,
+                                     num_experts, experts_per_token, _stream(stream)))
+
+
+def softmax(x, batch_size, size, stream=None):
+    """src/hip/softmax.hip:46 — in place."""
+    _check("moe_softmax", _lib.moe_softmax(_ptr(x), batch_size, size, _stream(stream)))
+
+
+def bucket_by_expert(topk_i, topk_v, B, K, E, expert_offsets, tokens_flat, weights_flat, slot_of=None, stream=None):
+    """src/hip/scheduler.hip:11-61 in one launch (count, scan, compaction)."""
+    _check("moe_bucket_by_expert",
+           _lib.moe_bucket_by_expert(_ptr(topk_i), _ptr(topk_v), B, K, E, _ptr(expert_offsets), _ptr(tokens_flat),
+                                     _ptr(weights_flat), _ptr(slot_of), _stream(stream)))
+
+
+def gather_rows(X, idx, Y, rows, H, stream=None):
+    """src/hip/scheduler.hip:63-85."""
+    _check("moe_gather_rows", _lib.moe_gather_rows(_ptr(X), _ptr(idx), _ptr(Y), rows, H, _stream(stream)))
+
+
+def build_work_queue(expert_offsets, E, work_queue, work_count, stream=None):
+    """src/hip/scheduler.hip:112-184 (single queue)."""
+    _check("moe_build_work_queue",
+           _lib.moe_build_work_queue(_ptr(expert_offsets), E, _ptr(work_queue), _ptr(work_count), _stream(stream)))
+
+
+def moe_mlp1_swiglu(work_queue, work_start, work_count, x_by_expert, gate_by_expert, weights_base, bias_base, H, I,
+                    expert_weight_stride, expert_bias_stride, alpha, swiglu_limit, maxNe, grid_cap, stream=None):
+    """src/hip/moe.hip:237."""
+    _check("moe_mlp1_swiglu",
+           _lib.moe_mlp1_swiglu(_ptr(work_queue), work_start, work_count, _ptr(x_by_expert), _ptr(gate_by_expert),
+                                _ptr(weights_base), _ptr(bias_base), H, I, expert_weight_stride, expert_bias_stride,
+                                alpha, swiglu_limit, maxNe, grid_cap, _stream(stream)))
+
+
+def moe_mlp2_scatter(work_queue, work_start, work_count, gate_by_expert, tokens_flat, weights_flat, e_agg,
+                     weights_base, bias_base, I, H, expert_weight_stride, expert_bias_stride, maxNe, grid_cap,
+                     stream=None):
+    """src/hip/moe.hip:514."""
+    _check("moe_mlp2_scatter",
+           _lib.moe_mlp2_scatter(_ptr(work_queue), work_start, work_count, _ptr(gate_by_expert), _ptr(tokens_flat),
+                                 _ptr(weights_flat), _ptr(e_agg), _ptr(weights_base), _ptr(bias_base), I, H,
+                                 expert_weight_stride, expert_bias_stride, maxNe, grid_cap, _stream(stream)))
+
+
+def moe_mlp1_swiglu_mxfp4(work_queue, work_start, work_count, x_by_expert, gate_by_expert, tiled_blocks,
+                          tiled_scales, bias_base, H, I, expert_bias_stride, alpha, swiglu_limit, maxNe, grid_cap,
+                          stream=None):
+    _check("moe_mlp1_swiglu_mxfp4",
+           _lib.moe_mlp1_swiglu_mxfp4(_ptr(work_queue), work_start, work_count, _ptr(x_by_expert),
+                                      _ptr(gate_by_expert), _ptr(tiled_blocks), _ptr(tiled_scales), _ptr(bias_base),
+                                      H, I, expert_bias_stride, alpha, swiglu_limit, maxNe, grid_cap,
+                                      _stream(stream)))
+
+
+def moe_mlp2_scatter_mxfp4(work_queue, work_start, work_count, gate_by_expert, tokens_flat, weights_flat, e_agg,
+                           tiled_blocks, tiled_scales, bias_base, I, H, expert_bias_stride, maxNe, grid_cap,
+                           stream=None):
+    _check("moe_mlp2_scatter_mxfp4",
+           _lib.moe_mlp2_scatter_mxfp4(_ptr(work_queue), work_start, work_count, _ptr(gate_by_expert),
+                                       _ptr(tokens_flat), _ptr(weights_flat), _ptr(e_agg), _ptr(tiled_blocks),
+                                       _ptr(tiled_scales), _ptr(bias_base), I, H, expert_bias_stride, maxNe,
+                                       grid_cap, _stream(stream)))
+
+
+def vecadd_and_zero(a, b, weight, batch, size, stream=None):
+    """src/hip/vecadd.hip:32."""
+    _check("moe_vecadd_and_zero", _lib.moe_vecadd_and_zero(_ptr(a), _ptr(b), weight, batch, size, _stream(stream)))
+
+
+def rmsnorm(o, x, weight, batch, size, stream=None):
+    """src/hip/rmsnorm.hip:39 (batched)."""
+    _check("moe_rmsnorm", _lib.moe_rmsnorm(_ptr(o), _ptr(x), _ptr(weight), batch, size, _stream(stream)))
+
+
+# ---- MXFP4 -------------------------------------------------------------------------------------
+def dequant_mxfp4(blocks, scales, out=None, stream=None):
+    """blocks [..., G, 16] u8, scales [..., G] u8 -> bf16 [..., G*32]
+    (tools/model_export/gpt-oss-20b/export_model_bin.py:95-133)."""
+    n_blocks = scales.numel()
+    if out is None:
+        out = torch.empty(tuple(scales.shape[:-1]) + (scales.shape[-1] * 32,), dtype=torch.bfloat16,
+                          device=blocks.device)
+    _check("moe_dequant_mxfp4", _lib.moe_dequant_mxfp4(_ptr(blocks), _ptr(scales), n_blocks, _ptr(out),
+                                                       _stream(stream)))
+    return out
+
+
+def mxfp4_tiled_bytes(rows, K):
+    bb, sb = _sz(0), _sz(0)
+    _lib.moe_mxfp4_tiled_bytes(rows, K, ctypes.byref(bb), ctypes.byref(sb))
+    return bb.value, sb.value
+
+
+def mxfp4_repack(blocks, scales, stream=None):
+    """blocks [E, rows, G, 16], scales [E, rows, G] -> (tiled_blocks, tiled_scales) u8 tensors."""
+    E, rows, G = scales.shape
+    bb, sb = mxfp4_tiled_bytes(rows, G * 32)
+    if bb == 0:
+        raise MoeError("moe_mxfp4_tiled_bytes", -2)
+    tb = torch.empty(E * bb, dtype=torch.uint8, device=blocks.device)
+    ts = torch.empty(E * sb, dtype=torch.uint8, device=blocks.device)
+    _check("moe_mxfp4_repack", _lib.moe_mxfp4_repack(_ptr(blocks), _ptr(scales), E, rows, G * 32, _ptr(tb), _ptr(ts),
+                                                     _stream(stream)))
+    return tb, ts
+
+
+def mxfp4_unpack(tiled_blocks, tiled_scales, E, rows, K, stream=None):
+    G = K // 32
+    blocks = torch.empty((E, rows, G, 16), dtype=torch.uint8, device=tiled_blocks.device)
+    scales = torch.empty((E, rows, G), dtype=torch.uint8, device=tiled_blocks.device)
+    _check("moe_mxfp4_unpack", _lib.moe_mxfp4_unpack(_ptr(tiled_blocks), _ptr(tiled_scales), E, rows, K, _ptr(blocks),
+                                                     _ptr(scales), _stream(stream)))
+    return blocks, scales
+
+
+def mxfp4_tiled_to_bf16(tiled_blocks, tiled_scales, E, rows, K, stream=None):
+    out = torch.empty((E, rows, K), dtype=torch.bfloat16, device=tiled_blocks.device)
+    _check("moe_mxfp4_tiled_to_bf16", _lib.moe_mxfp4_tiled_to_bf16(_ptr(tiled_blocks), _ptr(tiled_scales), E, rows, K,
+                                                                   _ptr(out), _stream(stream)))
+    return out
+
+
+# ---- whole block -------------------------------------------------------------------------------
+def block_workspace_bytes(T, H, I, E, K):
+    return _lib.moe_block_workspace_bytes(T, H, I, E, K)
+
+
+class MoeBlock:
+    """One layer's MoE weights plus a workspace sized for up to `max_tokens`; `forward` runs
+    router -> top-k -> softmax -> bucketing -> experts -> combine (src/forward.cpp:317-514)."""
+
+    def __init__(self, H, I, E, K, w_router, b_router, w_mlp1, b_mlp1, w_mlp2, b_mlp2, max_tokens,
+                 w_mlp1_scales=None, w_mlp2_scales=None, swiglu_limit=7.0, alpha=1.702):
+        self.H, self.I, self.E, self.K = H, I, E, K
+        self.fmt = MOE_WEIGHTS_BF16 if w_mlp1_scales is None else MOE_WEIGHTS_MXFP4_TILED
+        self.tensors = dict(w_router=w_router, b_router=b_router, w_mlp1=w_mlp1, b_mlp1=b_mlp1, w_mlp2=w_mlp2,
+                            b_mlp2=b_mlp2, w_mlp1_scales=w_mlp1_scales, w_mlp2_scales=w_mlp2_scales)
+        self.swiglu_limit, self.alpha = swiglu_limit, alpha
+        self.max_tokens = max_tokens
+        nbytes = block_workspace_bytes(max_tokens, H, I, E, K)
+        if nbytes == 0:
+            raise MoeError("moe_block_workspace_bytes", -2)
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=w_router.device)
+
+    def params(self, t, e_agg, topk_i, topk_v, router_score=None, residual_x=None, flags=0):
+        T = t.shape[0]
+        p = BlockParams()
+        p.struct_bytes = ctypes.sizeof(BlockParams)
+        p.n_tokens, p.hidden_dim, p.intermediate_dim = T, self.H, self.I
+        p.n_experts, p.experts_per_token, p.weight_format = self.E, self.K, self.fmt
+        p.swiglu_limit, p.alpha = self.swiglu_limit, self.alpha
+        p.t = _ptr(t)
+        for k, v in self.tensors.items():
+            setattr(p, k, _ptr(v))
+        p.e_agg, p.topk_i, p.topk_v = _ptr(e_agg), _ptr(topk_i), _ptr(topk_v)
+        p.router_score, p.residual_x = _ptr(router_score), _ptr(residual_x)
+        p.workspace, p.workspace_bytes = _ptr(self.workspace), self.workspace.numel()
+        p.flags = flags
+        return p
+
+    def forward(self, t, e_agg=None, topk_i=None, topk_v=None, router_score=None, residual_x=None, flags=0,
+                stream=None):
+        T = t.shape[0]
+        dev = t.device
+        if e_agg is None:
+            e_agg = torch.empty((T, self.H), dtype=torch.float32, device=dev)
+        if topk_i is None:
+            topk_i = torch.empty((T, self.K), dtype=torch.int32, device=dev)
+        if topk_v is None:
+            topk_v = torch.empty((T, self.K), dtype=torch.float32, device=dev)
+        p = self.params(t, e_agg, topk_i, topk_v, router_score, residual_x, flags)
+        _check("moe_block_forward", _lib.moe_block_forward(ctypes.byref(p), _stream(stream)))
+        return e_agg, topk_i, topk_v
+
+    def launch(self, p, stream):
+        """Re-issue a prepared parameter block (benchmark loop: no Python-side tensor work)."""
+        rc = _lib.moe_block_forward(ctypes.byref(p), stream)
+        if rc:
+            raise MoeError("moe_block_forward", rc)
+
+
+# ---- synthetic workloads (include/moe_synth.h) --------------------------------------------------
+def synth_normal_f32(dst, table_d, scale, seed, tensor_id, stream=None):
+    _check("moe_synth_normal_f32", _lib.moe_synth_normal_f32(_ptr(dst), dst.numel(), _ptr(table_d), scale, seed,
+                                                             tensor_id, _stream(stream)))
+
+
+def synth_normal_bf16(dst, table_d, scale, seed, tensor_id, stream=None):
+    _check("moe_synth_normal_bf16", _lib.moe_synth_normal_bf16(_ptr(dst), dst.numel(), _ptr(table_d), scale, seed,
+                                                               tensor_id, _stream(stream)))
+
+
+def synth_bytes(dst, seed, tensor_id, stream=None):
+    _check("moe_synth_bytes", _lib.moe_synth_bytes(_ptr(dst), dst.numel(), seed, tensor_id, _stream(stream)))
+
+
+def synth_range_bytes(dst, seed, tensor_id, lo, span, stream=None):
+    _check("moe_synth_range_bytes", _lib.moe_synth_range_bytes(_ptr(dst), dst.numel(), seed, tensor_id, lo, span,
+                                                               _stream(stream)))

@@ -1,0 +1,431 @@
+// extern "C" entry points of libmoe_gfx950.so (declared in include/moe_abi.h): argument checks,
+// workspace carving and launch sequencing.  No entry allocates, synchronises or exits.
+#include "common.h"
+#include "kernels.h"
+
+using namespace moe;
+
+namespace {
+
+constexpr size_t kAlign = 256;
+inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+inline hipStream_t as_stream(moe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Token-block size of the expert kernels' tile map.
+constexpr int kStreamTileTokens = 64;
+
+// Carves the caller's workspace for moe_block_forward; with base == nullptr only sizes it.
+struct BlockWorkspace {
+    double* router_partial;
+    uint16_t* t_bf16;      // [T,H] bf16 copy of the block input
+    int* expert_offsets;   // [E+1]
+    int* tokens_flat;      // [A]
+    float* weights_flat;   // [A]
+    int* slot_of;          // [A]
+    int* tile_expert;      // [max_tiles]
+    int* tile_row0;
+    int* tile_rows;
+    int* n_tiles;          // [1]
+    uint16_t* h_by_slot;   // [A, I] bf16 SwiGLU outputs
+    float* y_by_slot;      // [A, H] fp32 down-projection rows
+    int max_tiles;
+    size_t bytes;
+
+    BlockWorkspace(void* base, int T, int H, int I, int E, int K) {
+        const size_t A = (size_t)T * K;
+        size_t off = 0;
+        auto take = [&](size_t n) {
+            void* p = base ? static_cast<char*>(base) + off : nullptr;
+            off += align_up(n);
+            return p;
+        };
+        const int S = router_segments(T, E, H, false);
+        router_partial = static_cast<double*>(take((size_t)S * T * E * sizeof(double)));
+        t_bf16 = static_cast<uint16_t*>(take((size_t)T * H * 2));
+        expert_offsets = static_cast<int*>(take((size_t)(E + 1) * 4));
+        tokens_flat = static_cast<int*>(take(A * 4));
+        weights_flat = static_cast<float*>(take(A * 4));
+        slot_of = static_cast<int*>(take(A * 4));
+        max_tiles = tile_map_capacity((int)A, E, kStreamTileTokens);
+        tile_expert = static_cast<int*>(take((size_t)max_tiles * 4));
+        tile_row0 = static_cast<int*>(take((size_t)max_tiles * 4));
+        tile_rows = static_cast<int*>(take((size_t)max_tiles * 4));
+        n_tiles = static_cast<int*>(take(4));
+        h_by_slot = static_cast<uint16_t*>(take(A * I * 2));
+        y_by_slot = static_cast<float*>(take(A * H * 4));
+        bytes = off;
+    }
+};
+
+int check_dims(int T, int H, int I, int E, int K) {
+    if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || K <= 0) return MOE_ERR_SHAPE;
+    if (H % 64 != 0 || I % 64 != 0) return MOE_ERR_SHAPE;
+    if (K > E) return MOE_ERR_SHAPE;
+    if (E > 1024 || K > 8) return MOE_ERR_LIMIT;
+    if ((long long)T * K > 0x7FFFFFFFll / 4) return MOE_ERR_LIMIT;
+    return MOE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int moe_abi_version(void) { return MOE_ABI_VERSION; }
+
+const char* moe_error_string(int code) {
+    switch (code) {
+        case MOE_OK: return "ok";
+        case MOE_ERR_NULL: return "a required pointer is NULL";
+        case MOE_ERR_SHAPE: return "a dimension is non-positive or not a documented multiple";
+        case MOE_ERR_LIMIT: return "a dimension exceeds a documented maximum";
+        case MOE_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case MOE_ERR_FORMAT: return "unknown weight format or flag";
+        case MOE_ERR_ALIGN: return "a pointer does not have the documented alignment";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}
+
+// ---- router ----------------------------------------------------------------------------------
+size_t moe_router_scratch_bytes(int N, int M) {
+    if (N <= 0 || M <= 0) return 0;
+    return (size_t)16 * N * M * sizeof(double);
+}
+
+int moe_gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias, int N,
+                    int K, int M, void* scratch, size_t scratch_bytes, moe_stream_t stream) {
+    if (!xout || !x_batch || !w || !bias) return MOE_ERR_NULL;
+    if (N <= 0 || K <= 0 || M <= 0 || K % 8 != 0) return MOE_ERR_SHAPE;
+    if (M > 1024) return MOE_ERR_LIMIT;
+    const int S = router_segments(N, M, K, false);
+    if (!scratch || ((uintptr_t)scratch & 7u) || scratch_bytes < (size_t)S * N * M * sizeof(double))
+        return MOE_ERR_WORKSPACE;
+    double* partial = static_cast<double*>(scratch);
+    int rc = launch_router_partial(x_batch, w, partial, N, K, M, S, as_stream(stream));
+    if (rc) return rc;
+    return launch_router_finalize(partial, S, nullptr, bias, xout, nullptr, nullptr, N, M, 0, 0, 0, as_stream(stream));
+}
+
+int moe_topk(float* topk_values, int* topk_indices, const float* router_scores, int batch_size, int num_experts,
+             int experts_per_token, moe_stream_t stream) {
+    if (!topk_values || !topk_indices || !router_scores) return MOE_ERR_NULL;
+    if (batch_size <= 0 || num_experts <= 0 || experts_per_token <= 0 || experts_per_token > num_experts)
+        return MOE_ERR_SHAPE;
+    if (num_experts > 1024 || experts_per_token > 8) return MOE_ERR_LIMIT;
+    return launch_router_finalize(nullptr, 0, router_scores, nullptr, nullptr, topk_values, topk_indices, batch_size,
+                                  num_experts, experts_per_token, 1, 0, as_stream(stream));
+}
+
+int moe_softmax(float* x, int batch_size, int size, moe_stream_t stream) {
+    if (!x) return MOE_ERR_NULL;
+    if (batch_size <= 0 || size <= 0) return MOE_ERR_SHAPE;
+    if (size > 64) return MOE_ERR_LIMIT;
+    return launch_softmax_rows(x, batch_size, size, as_stream(stream));
+}
+
+// ---- bucketing -------------------------------------------------------------------------------
+int moe_bucket_by_expert(const int* topk_i, const float* topk_v, int B, int K, int E, int* expert_offsets,
+                         int* tokens_flat, float* weights_flat, int* slot_of, moe_stream_t stream) {
+    if (!topk_i || !topk_v || !expert_offsets || !tokens_flat || !weights_flat) return MOE_ERR_NULL;
+    if (B <= 0 || K <= 0 || E <= 0) return MOE_ERR_SHAPE;
+    if (E > 1024 || (long long)B * K > 0x7FFFFFFFll / 4) return MOE_ERR_LIMIT;
+    TileMap none{nullptr, nullptr, nullptr, nullptr, 0, 0};
+    return launch_bucket(topk_i, topk_v, B, K, E, expert_offsets, tokens_flat, weights_flat, slot_of, none,
+                         as_stream(stream));
+}
+
+int moe_gather_rows(const float* X, const int* idx, float* Y, int rows, int H, moe_stream_t stream) {
+    if (!X || !idx || !Y) return MOE_ERR_NULL;
+    if (rows <= 0 || H <= 0 || H % 4 != 0) return MOE_ERR_SHAPE;
+    if (rows > 65535) {
+        // grid.y limit: split into slabs
+        for (int r0 = 0; r0 < rows; r0 += 65535) {
+            int rc = launch_gather_rows(X, idx + r0, Y + (size_t)r0 * H, rows - r0 < 65535 ? rows - r0 : 65535, H,
+                                        as_stream(stream));
+            if (rc) return rc;
+        }
+        return MOE_OK;
+    }
+    return launch_gather_rows(X, idx, Y, rows, H, as_stream(stream));
+}
+
+int moe_build_work_queue(const int* expert_offsets, int E, int* work_queue, int* work_count, moe_stream_t stream) {
+    if (!expert_offsets || !work_queue || !work_count) return MOE_ERR_NULL;
+    if (E <= 0) return MOE_ERR_SHAPE;
+    return launch_build_work_queue(expert_offsets, E, work_queue, work_count, as_stream(stream));
+}
+
+// ---- expert GEMMs, reference data flow ---------------------------------------------------------
+static int queue_gemm(int epi, int format, const int* work_queue, int work_start, int work_count,
+                      const float* act, void* out, const int* tokens_flat, const float* weights_flat,
+                      const void* w, const uint8_t* w_scales, const moe_bf16_t* bias, int rows, int Kdim,
+                      long long w_stride, long long s_stride, long long bias_stride, float alpha, float limit,
+                      int maxNe, moe_stream_t stream) {
+    if (!work_queue || !act || !out || !w || !bias) return MOE_ERR_NULL;
+    if (format == MOE_WEIGHTS_MXFP4_TILED && !w_scales) return MOE_ERR_NULL;
+    if (work_count < 0 || work_start < 0 || rows <= 0 || Kdim <= 0) return MOE_ERR_SHAPE;
+    if (work_count > 65535) return MOE_ERR_LIMIT;
+    ExpertGemmArgs a{};
+    a.w = w;
+    a.w_scales = w_scales;
+    a.bias = bias;
+    a.act_f32 = act;
+    a.tokens_flat = tokens_flat;
+    a.weights_flat = weights_flat;
+    a.work_queue = work_queue;
+    a.work_start = work_start;
+    a.work_count = work_count;
+    a.max_rows_hint = maxNe < 64 ? 64 : (maxNe > 64 * 1024 ? 64 * 1024 : maxNe);
+    a.out = out;
+    a.rows = rows;
+    a.K = Kdim;
+    a.w_expert_stride = w_stride;
+    a.s_expert_stride = s_stride;
+    a.bias_expert_stride = bias_stride;
+    a.alpha = alpha;
+    a.limit = limit;
+    a.format = format;
+    return launch_expert_stream(a, epi, as_stream(stream));
+}
+
+int moe_mlp1_swiglu(const int* work_queue, int work_start, int work_count, const float* x_by_expert,
+                    float* gate_by_expert, const moe_bf16_t* weights_base, const moe_bf16_t* bias_base, int H, int I,
+                    long long expert_weight_stride, long long expert_bias_stride, float alpha, float swiglu_limit,
+                    int maxNe, int grid_cap, moe_stream_t stream) {
+    (void)grid_cap;
+    if (H % 64 != 0 || I % 32 != 0) return MOE_ERR_SHAPE;
+    return queue_gemm(2, MOE_WEIGHTS_BF16, work_queue, work_start, work_count, x_by_expert, gate_by_expert, nullptr,
+                      nullptr, weights_base, nullptr, bias_base, 2 * I, H, expert_weight_stride, 0,
+                      expert_bias_stride, alpha, swiglu_limit, maxNe, stream);
+}
+
+int moe_mlp2_scatter(const int* work_queue, int work_start, int work_count, const float* gate_by_expert,
+                     const int* tokens_flat, const float* weights_flat, float* e_agg,
+                     const moe_bf16_t* weights_base, const moe_bf16_t* bias_base, int I, int H,
+                     long long expert_weight_stride, long long expert_bias_stride, int maxNe, int grid_cap,
+                     moe_stream_t stream) {
+    (void)grid_cap;
+    if (!tokens_flat || !weights_flat) return MOE_ERR_NULL;
+    if (H % 64 != 0 || I % 64 != 0) return MOE_ERR_SHAPE;
+    return queue_gemm(3, MOE_WEIGHTS_BF16, work_queue, work_start, work_count, gate_by_expert, e_agg, tokens_flat,
+                      weights_flat, weights_base, nullptr, bias_base, H, I, expert_weight_stride, 0,
+                      expert_bias_stride, 0.f, 0.f, maxNe, stream);
+}
+
+int moe_mlp1_swiglu_mxfp4(const int* work_queue, int work_start, int work_count, const float* x_by_expert,
+                          float* gate_by_expert, const uint8_t* tiled_blocks, const uint8_t* tiled_scales,
+                          const moe_bf16_t* bias_base, int H, int I, long long expert_bias_stride, float alpha,
+                          float swiglu_limit, int maxNe, int grid_cap, moe_stream_t stream) {
+    (void)grid_cap;
+    if (H % 32 != 0 || I % 32 != 0 || H <= 0 || I <= 0) return MOE_ERR_SHAPE;
+    size_t bb, sb;
+    mxfp4_tiled_bytes(2 * I, H, &bb, &sb);
+    return queue_gemm(2, MOE_WEIGHTS_MXFP4_TILED, work_queue, work_start, work_count, x_by_expert, gate_by_expert,
+                      nullptr, nullptr, tiled_blocks, tiled_scales, bias_base, 2 * I, H, (long long)bb, (long long)sb,
+                      expert_bias_stride, alpha, swiglu_limit, maxNe, stream);
+}
+
+int moe_mlp2_scatter_mxfp4(const int* work_queue, int work_start, int work_count, const float* gate_by_expert,
+                           const int* tokens_flat, const float* weights_flat, float* e_agg,
+                           const uint8_t* tiled_blocks, const uint8_t* tiled_scales, const moe_bf16_t* bias_base,
+                           int I, int H, long long expert_bias_stride, int maxNe, int grid_cap, moe_stream_t stream) {
+    (void)grid_cap;
+    if (!tokens_flat || !weights_flat) return MOE_ERR_NULL;
+    if (H % 64 != 0 || I % 32 != 0 || H <= 0 || I <= 0) return MOE_ERR_SHAPE;
+    size_t bb, sb;
+    mxfp4_tiled_bytes(H, I, &bb, &sb);
+    return queue_gemm(3, MOE_WEIGHTS_MXFP4_TILED, work_queue, work_start, work_count, gate_by_expert, e_agg,
+                      tokens_flat, weights_flat, tiled_blocks, tiled_scales, bias_base, H, I, (long long)bb,
+                      (long long)sb, expert_bias_stride, 0.f, 0.f, maxNe, stream);
+}
+
+int moe_vecadd_and_zero(float* a, float* b, float weight, int batch, int size, moe_stream_t stream) {
+    if (!a || !b) return MOE_ERR_NULL;
+    if (batch <= 0 || size <= 0) return MOE_ERR_SHAPE;
+    return launch_vecadd_and_zero(a, b, weight, batch, size, as_stream(stream));
+}
+
+int moe_rmsnorm(float* o, const float* x, const moe_bf16_t* weight, int batch, int size, moe_stream_t stream) {
+    if (!o || !x || !weight) return MOE_ERR_NULL;
+    if (batch <= 0 || size <= 0) return MOE_ERR_SHAPE;
+    return launch_rmsnorm(o, x, weight, batch, size, as_stream(stream));
+}
+
+// ---- MXFP4 -----------------------------------------------------------------------------------
+int moe_dequant_mxfp4(const uint8_t* blocks, const uint8_t* scales, long long n_blocks, moe_bf16_t* out,
+                      moe_stream_t stream) {
+    if (!blocks || !scales || !out) return MOE_ERR_NULL;
+    if (n_blocks <= 0) return MOE_ERR_SHAPE;
+    if (n_blocks > 0x7FFFFFFFll * 256) return MOE_ERR_LIMIT;
+    if (((uintptr_t)blocks | (uintptr_t)out) & 15u) return MOE_ERR_ALIGN;
+    return launch_dequant_mxfp4(blocks, scales, n_blocks, out, as_stream(stream));
+}
+
+void moe_mxfp4_tiled_bytes(int rows, int K, size_t* block_bytes_per_expert, size_t* scale_bytes_per_expert) {
+    if (rows <= 0 || K <= 0 || rows % 64 != 0 || K % 32 != 0) {
+        if (block_bytes_per_expert) *block_bytes_per_expert = 0;
+        if (scale_bytes_per_expert) *scale_bytes_per_expert = 0;
+        return;
+    }
+    mxfp4_tiled_bytes(rows, K, block_bytes_per_expert, scale_bytes_per_expert);
+}
+
+static int repack_common(const uint8_t* blocks, const uint8_t* scales, int E, int rows, int K, uint8_t* tiled_blocks,
+                         uint8_t* tiled_scales, bool inverse, moe_stream_t stream) {
+    if (!blocks || !scales || !tiled_blocks || !tiled_scales) return MOE_ERR_NULL;
+    if (E <= 0 || rows <= 0 || K <= 0 || rows % 64 != 0 || K % 32 != 0) return MOE_ERR_SHAPE;
+    if (((uintptr_t)blocks | (uintptr_t)tiled_blocks) & 15u) return MOE_ERR_ALIGN;
+    if ((uintptr_t)tiled_scales & 3u) return MOE_ERR_ALIGN;
+    if ((long long)E * rows * (K / 32) > 0x7FFFFFFFll * 256) return MOE_ERR_LIMIT;
+    return launch_mxfp4_repack(blocks, scales, E, rows, K, tiled_blocks, tiled_scales, inverse, as_stream(stream));
+}
+
+int moe_mxfp4_repack(const uint8_t* blocks, const uint8_t* scales, int E, int rows, int K, uint8_t* tiled_blocks,
+                     uint8_t* tiled_scales, moe_stream_t stream) {
+    return repack_common(blocks, scales, E, rows, K, tiled_blocks, tiled_scales, false, stream);
+}
+
+int moe_mxfp4_unpack(const uint8_t* tiled_blocks, const uint8_t* tiled_scales, int E, int rows, int K,
+                     uint8_t* blocks, uint8_t* scales, moe_stream_t stream) {
+    return repack_common(blocks, scales, E, rows, K, const_cast<uint8_t*>(tiled_blocks),
+                         const_cast<uint8_t*>(tiled_scales), true, stream);
+}
+
+int moe_mxfp4_tiled_to_bf16(const uint8_t* tiled_blocks, const uint8_t* tiled_scales, int E, int rows, int K,
+                            moe_bf16_t* out, moe_stream_t stream) {
+    if (!tiled_blocks || !tiled_scales || !out) return MOE_ERR_NULL;
+    if (E <= 0 || rows <= 0 || K <= 0 || rows % 64 != 0 || K % 32 != 0) return MOE_ERR_SHAPE;
+    if (((uintptr_t)tiled_blocks | (uintptr_t)out) & 15u) return MOE_ERR_ALIGN;
+    return launch_mxfp4_tiled_to_bf16(tiled_blocks, tiled_scales, E, rows, K, out, as_stream(stream));
+}
+
+// ---- whole block -----------------------------------------------------------------------------
+size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int intermediate_dim, int n_experts,
+                                 int experts_per_token) {
+    if (check_dims(n_tokens, hidden_dim, intermediate_dim, n_experts, experts_per_token) != MOE_OK) return 0;
+    return BlockWorkspace(nullptr, n_tokens, hidden_dim, intermediate_dim, n_experts, experts_per_token).bytes;
+}
+
+int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
+    if (!p) return MOE_ERR_NULL;
+    if (p->struct_bytes != sizeof(moe_block_params)) return MOE_ERR_FORMAT;
+    const int T = p->n_tokens, H = p->hidden_dim, I = p->intermediate_dim, E = p->n_experts,
+              K = p->experts_per_token;
+    int rc = check_dims(T, H, I, E, K);
+    if (rc) return rc;
+    if (!p->t || !p->w_router || !p->b_router || !p->w_mlp1 || !p->b_mlp1 || !p->w_mlp2 || !p->b_mlp2 ||
+        !p->e_agg || !p->topk_i || !p->topk_v)
+        return MOE_ERR_NULL;
+    const int fmt = p->weight_format;
+    if (fmt != MOE_WEIGHTS_BF16 && fmt != MOE_WEIGHTS_MXFP4_TILED) return MOE_ERR_FORMAT;
+    if (fmt == MOE_WEIGHTS_MXFP4_TILED && (!p->w_mlp1_scales || !p->w_mlp2_scales)) return MOE_ERR_NULL;
+    if (((uintptr_t)p->t | (uintptr_t)p->e_agg | (uintptr_t)p->w_mlp1 | (uintptr_t)p->w_mlp2 |
+         (uintptr_t)p->w_router | (uintptr_t)p->residual_x) & 15u)
+        return MOE_ERR_ALIGN;
+    if (!p->workspace || ((uintptr_t)p->workspace & (kAlign - 1))) return MOE_ERR_WORKSPACE;
+    BlockWorkspace ws(p->workspace, T, H, I, E, K);
+    if (p->workspace_bytes < ws.bytes) return MOE_ERR_WORKSPACE;
+    hipStream_t stream = as_stream(stream_);
+
+    // 1. router logits -> top-k -> softmax  (src/forward.cpp:318-327; src/run.cpp:630-642)
+    const int S = router_segments(T, E, H, (p->flags & MOE_FLAG_ROUTER_STRICT_ORDER) != 0);
+    rc = launch_router_partial(p->t, p->w_router, ws.router_partial, T, H, E, S, stream);
+    if (rc) return rc;
+    rc = launch_router_finalize(ws.router_partial, S, nullptr, p->b_router, p->router_score, p->topk_v, p->topk_i, T, E,
+                                K, 1, 1, stream);
+    if (rc) return rc;
+    rc = launch_convert_f32_bf16(p->t, ws.t_bf16, (size_t)T * H, stream);
+    if (rc) return rc;
+
+    // 2. bucketing + token-block map  (src/forward.cpp:329-376)
+    TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, kStreamTileTokens, ws.max_tiles};
+    rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat, ws.slot_of,
+                       map, stream);
+    if (rc) return rc;
+
+    // 3. gate/up GEMM + SwiGLU  (src/forward.cpp:474-479; src/run.cpp:657-689)
+    ExpertGemmArgs g{};
+    g.tokens_flat = ws.tokens_flat;
+    g.tile_expert = ws.tile_expert;
+    g.tile_row0 = ws.tile_row0;
+    g.tile_rows = ws.tile_rows;
+    g.n_tiles = ws.n_tiles;
+    g.max_tiles = ws.max_tiles;
+    g.alpha = p->alpha;
+    g.limit = p->swiglu_limit;
+    g.format = fmt;
+
+    ExpertGemmArgs a1 = g;
+    a1.w = p->w_mlp1;
+    a1.w_scales = static_cast<const uint8_t*>(p->w_mlp1_scales);
+    a1.bias = p->b_mlp1;
+    a1.act = ws.t_bf16;
+    a1.gather = 1;
+    a1.out = ws.h_by_slot;
+    a1.rows = 2 * I;
+    a1.K = H;
+    a1.bias_expert_stride = 2LL * I;
+    if (fmt == MOE_WEIGHTS_BF16) {
+        a1.w_expert_stride = 2LL * I * H;
+    } else {
+        size_t bb, sb;
+        mxfp4_tiled_bytes(2 * I, H, &bb, &sb);
+        a1.w_expert_stride = (long long)bb;
+        a1.s_expert_stride = (long long)sb;
+    }
+    rc = launch_expert_stream(a1, 0, stream);
+    if (rc) return rc;
+
+    // 4. down GEMM  (src/forward.cpp:481-487; src/run.cpp:691-700)
+    ExpertGemmArgs a2 = g;
+    a2.w = p->w_mlp2;
+    a2.w_scales = static_cast<const uint8_t*>(p->w_mlp2_scales);
+    a2.bias = p->b_mlp2;
+    a2.act = ws.h_by_slot;
+    a2.gather = 0;
+    a2.out = ws.y_by_slot;
+    a2.rows = H;
+    a2.K = I;
+    a2.bias_expert_stride = H;
+    if (fmt == MOE_WEIGHTS_BF16) {
+        a2.w_expert_stride = (long long)H * I;
+    } else {
+        size_t bb, sb;
+        mxfp4_tiled_bytes(H, I, &bb, &sb);
+        a2.w_expert_stride = (long long)bb;
+        a2.s_expert_stride = (long long)sb;
+    }
+    rc = launch_expert_stream(a2, 1, stream);
+    if (rc) return rc;
+
+    // 5. weighted combine in ascending expert id (+ residual)  (src/run.cpp:702-712)
+    return launch_combine(ws.y_by_slot, ws.slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x, T, K, H, stream);
+}
+
+// ---- synthetic workloads ----------------------------------------------------------------------
+int moe_synth_normal_f32(float* dst, long long n, const float* table_d, float scale, unsigned seed,
+                         unsigned tensor_id, moe_stream_t stream) {
+    if (!dst || !table_d) return MOE_ERR_NULL;
+    if (n <= 0) return MOE_ERR_SHAPE;
+    return launch_synth(0, dst, n, table_d, scale, seed, tensor_id, 0, 0, as_stream(stream));
+}
+int moe_synth_normal_bf16(moe_bf16_t* dst, long long n, const float* table_d, float scale, unsigned seed,
+                          unsigned tensor_id, moe_stream_t stream) {
+    if (!dst || !table_d) return MOE_ERR_NULL;
+    if (n <= 0) return MOE_ERR_SHAPE;
+    return launch_synth(1, dst, n, table_d, scale, seed, tensor_id, 0, 0, as_stream(stream));
+}
+int moe_synth_bytes(uint8_t* dst, long long n, unsigned seed, unsigned tensor_id, moe_stream_t stream) {
+    if (!dst) return MOE_ERR_NULL;
+    if (n <= 0) return MOE_ERR_SHAPE;
+    if ((uintptr_t)dst & 3u) return MOE_ERR_ALIGN;
+    return launch_synth(2, dst, n, nullptr, 0.f, seed, tensor_id, 0, 0, as_stream(stream));
+}
+int moe_synth_range_bytes(uint8_t* dst, long long n, unsigned seed, unsigned tensor_id, unsigned lo, unsigned span,
+                          moe_stream_t stream) {
+    if (!dst) return MOE_ERR_NULL;
+    if (n <= 0 || span == 0 || lo + span > 256) return MOE_ERR_SHAPE;
+    if ((uintptr_t)dst & 3u) return MOE_ERR_ALIGN;
+    return launch_synth(3, dst, n, nullptr, 0.f, seed, tensor_id, lo, span, as_stream(stream));
+}
+
+}  // extern "C"

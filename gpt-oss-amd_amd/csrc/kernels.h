@@ -1,0 +1,85 @@
+// Internal launcher declarations shared by the translation units of libmoe_gfx950.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace moe {
+
+// ---- router.hip -------------------------------------------------------------------------------
+int router_segments(int T, int E, int H, bool strict);
+int launch_router_partial(const float* x, const uint16_t* w, double* partial, int T, int H, int E, int S,
+                          hipStream_t stream);
+int launch_router_finalize(const double* partial, int S, const float* scores_in, const uint16_t* bias,
+                           float* scores_out, float* topk_v, int* topk_i, int T, int E, int K, int do_topk,
+                           int do_softmax, hipStream_t stream);
+int launch_softmax_rows(float* x, int B, int size, hipStream_t stream);
+int launch_convert_f32_bf16(const float* in, uint16_t* out, size_t n, hipStream_t stream);
+
+// ---- bucket.hip -------------------------------------------------------------------------------
+// Token-block map consumed by the expert kernels: tile i covers rows
+// [tile_row0[i], tile_row0[i] + tile_rows[i]) of tokens_flat, all routed to tile_expert[i].
+struct TileMap {
+    int* tile_expert;
+    int* tile_row0;
+    int* tile_rows;
+    int* n_tiles;   // device scalar
+    int tile_tokens;  // rows per tile (NB); 0 = no map requested
+    int max_tiles;    // capacity = upper bound used as grid dimension
+};
+inline int tile_map_capacity(int A, int E, int tile_tokens) { return (A + tile_tokens - 1) / tile_tokens + E; }
+
+int launch_bucket(const int* topk_i, const float* topk_v, int T, int K, int E, int* expert_offsets,
+                  int* tokens_flat, float* weights_flat, int* slot_of, TileMap map, hipStream_t stream);
+int launch_gather_rows(const float* X, const int* idx, float* Y, int rows, int H, hipStream_t stream);
+int launch_build_work_queue(const int* expert_offsets, int E, int* work_queue, int* work_count,
+                            hipStream_t stream);
+
+// ---- experts_stream.hip ------------------------------------------------------------------------
+struct ExpertGemmArgs {
+    const void* w;              // bf16 [E, rows, K] or tiled MXFP4 blocks
+    const uint8_t* w_scales;    // tiled MXFP4 scales or nullptr
+    const uint16_t* bias;       // bf16 [E, rows]
+    const uint16_t* act;        // bf16 activations: [T, K] (gathered through tokens_flat) or [A, K]
+    const float* act_f32;       // queue entries only: fp32 activations [A, K] indexed by slot row
+    const int* tokens_flat;     // slot row -> token id
+    const float* weights_flat;  // slot row -> router weight (scatter epilogue)
+    int gather;                 // 1: activation row = tokens_flat[slot row]; 0: slot row itself
+    const int* work_queue;      // non-null: (expert, row_offset, row_count) triples instead of the tile map
+    int work_start, work_count, max_rows_hint;
+    const int* tile_expert;
+    const int* tile_row0;
+    const int* tile_rows;
+    const int* n_tiles;
+    void* out;                  // see launch_expert_stream
+    int rows;                   // weight rows per expert (2I or H)
+    int K;                      // contraction length (H or I)
+    long long w_expert_stride;  // bf16: elements; MXFP4: bytes of blocks per expert
+    long long s_expert_stride;  // MXFP4: bytes of scales per expert
+    long long bias_expert_stride;
+    float alpha, limit;
+    int max_tiles;
+    int format;
+};
+int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
+
+// ---- combine.hip -------------------------------------------------------------------------------
+int launch_combine(const float* y_by_slot, const int* slot_of, const int* topk_i, const float* topk_v,
+                   float* e_agg, float* residual_x, int T, int K, int H, hipStream_t stream);
+int launch_vecadd_and_zero(float* a, float* b, float weight, int batch, int size, hipStream_t stream);
+int launch_rmsnorm(float* o, const float* x, const uint16_t* weight, int batch, int size, hipStream_t stream);
+
+// ---- mxfp4.hip ---------------------------------------------------------------------------------
+void mxfp4_tiled_bytes(int rows, int K, size_t* block_bytes, size_t* scale_bytes);
+int launch_dequant_mxfp4(const uint8_t* blocks, const uint8_t* scales, long long n_blocks, uint16_t* out,
+                         hipStream_t stream);
+int launch_mxfp4_repack(const uint8_t* blocks, const uint8_t* scales, int E, int rows, int K,
+                        uint8_t* tiled_blocks, uint8_t* tiled_scales, bool inverse, hipStream_t stream);
+int launch_mxfp4_tiled_to_bf16(const uint8_t* tiled_blocks, const uint8_t* tiled_scales, int E, int rows, int K,
+                               uint16_t* out, hipStream_t stream);
+
+// ---- synth.hip ---------------------------------------------------------------------------------
+int launch_synth(int kind, void* dst, long long n, const float* table, float scale, unsigned seed,
+                 unsigned tensor_id, unsigned lo, unsigned span, hipStream_t stream);
+
+}  // namespace moe

@@ -1,0 +1,272 @@
+// Router: logits (fp32 products, fp64 accumulation) -> top-k (ties to the lower expert id) ->
+// softmax over the k selected logits.  Arithmetic follows the reference CPU path
+// (src/run.cpp:321-404, 628-642); the GPU functions replaced are gemm_router
+// (src/hip/gemms/gemm_router.hip:184), topk (src/hip/topk.hip:59) and softmax (src/hip/softmax.hip:46).
+#include "common.h"
+#include "kernels.h"
+
+namespace moe {
+
+// ---------------------------------------------------------------------------------------------
+// Partial dot products.  One lane = one token, one wave = EG experts over one k-segment, so every
+// accumulator walks its segment in ascending k exactly like the reference loop; with one segment
+// the fp64 sum is bit-identical to src/run.cpp:348-351.  The four waves of a block share a
+// transposed activation chunk in LDS (row stride 65 floats: conflict-free for the transposing
+// store and for the lane-per-token read); weights are wave-uniform 16-byte loads.
+// grid = (ceil(T/64), ceil(E/(4*EG)), S), block = 256.
+// partial layout: [S][T][E] fp64.
+// ---------------------------------------------------------------------------------------------
+template <int EG>
+__global__ __launch_bounds__(256) void router_partial_kernel(const float* __restrict__ x,
+                                                             const uint16_t* __restrict__ w,
+                                                             double* __restrict__ partial, int T, int H,
+                                                             int E, int seg_len) {
+    constexpr int KC = 64;
+    __shared__ float xs[KC][65];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t0 = blockIdx.x * 64;
+    const int e0 = (blockIdx.y * 4 + wave) * EG;
+    const int s = blockIdx.z;
+    const int kbeg = s * seg_len;
+    const int kend = min(H, kbeg + seg_len);
+
+    double acc[EG];
+#pragma unroll
+    for (int j = 0; j < EG; ++j) acc[j] = 0.0;
+
+    for (int k0 = kbeg; k0 < kend; k0 += KC) {
+        const int kc = min(KC, kend - k0);  // multiple of 8
+        const int q4 = kc >> 2;
+        for (int i = threadIdx.x; i < 64 * q4; i += 256) {
+            const int tl = i / q4;
+            const int c = i - tl * q4;
+            const int tok = t0 + tl;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (tok < T) v = *reinterpret_cast<const float4*>(x + (size_t)tok * H + k0 + 4 * c);
+            xs[4 * c + 0][tl] = v.x;
+            xs[4 * c + 1][tl] = v.y;
+            xs[4 * c + 2][tl] = v.z;
+            xs[4 * c + 3][tl] = v.w;
+        }
+        __syncthreads();
+        if (e0 < E) {
+            for (int kk = 0; kk < kc; kk += 8) {
+                uint4 wv[EG];
+#pragma unroll
+                for (int j = 0; j < EG; ++j) {
+                    const int e = min(e0 + j, E - 1);
+                    wv[j] = *reinterpret_cast<const uint4*>(w + (size_t)e * H + k0 + kk);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float xv = xs[kk + i][lane];
+#pragma unroll
+                    for (int j = 0; j < EG; ++j) {
+                        const uint32_t word = (i < 2) ? wv[j].x : (i < 4) ? wv[j].y : (i < 6) ? wv[j].z : wv[j].w;
+                        const float wf = (i & 1) ? __uint_as_float(word & 0xFFFF0000u)
+                                                 : __uint_as_float(word << 16);
+                        acc[j] += (double)__fmul_rn(wf, xv);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    const int tok = t0 + lane;
+    if (tok < T) {
+#pragma unroll
+        for (int j = 0; j < EG; ++j) {
+            const int e = e0 + j;
+            if (e < E) partial[((size_t)s * T + tok) * E + e] = acc[j];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Finalise: one wave per token.  score[e] = float(sum_s partial[s][t][e]) + bias[e]
+// (src/run.cpp:352, 635-637), then K rounds of wave-wide argmax ordered by (value desc, index
+// asc), then the softmax of src/run.cpp:321-339 on the K selected values.
+// When `partial` is NULL the scores are read from `scores_in` instead.
+// grid = ceil(T/4), block = 256, dynamic LDS = 4*E floats.
+// ---------------------------------------------------------------------------------------------
+MOE_DEVICE bool better(float va, int ia, float vb, int ib) { return va > vb || (va == vb && ia < ib); }
+
+__global__ __launch_bounds__(256) void router_finalize_kernel(const double* __restrict__ partial, int S,
+                                                              const float* __restrict__ scores_in,
+                                                              const uint16_t* __restrict__ bias,
+                                                              float* __restrict__ scores_out,
+                                                              float* __restrict__ topk_v,
+                                                              int* __restrict__ topk_i, int T, int E,
+                                                              int K, int do_topk, int do_softmax) {
+    extern __shared__ float sc[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= T) return;  // no block-wide barrier below
+    float* my = sc + (size_t)wave * E;
+
+    for (int e = lane; e < E; e += 64) {
+        float v;
+        if (partial) {
+            double sum = 0.0;
+            for (int s = 0; s < S; ++s) sum += partial[((size_t)s * T + t) * E + e];
+            v = (float)sum;
+            v += bf16_bits_to_f32(bias[e]);
+        } else {
+            v = scores_in[(size_t)t * E + e];
+        }
+        my[e] = v;
+        if (scores_out) scores_out[(size_t)t * E + e] = v;
+    }
+    if (!do_topk) return;
+    __builtin_amdgcn_wave_barrier();
+
+    uint32_t taken = 0;  // bit c set: candidate lane + 64*c already selected
+    float sel_v[8];
+    int sel_i[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        sel_v[r] = 0.f;
+        sel_i[r] = 0;
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        if (r < K) {
+            float bv = -INFINITY;
+            int bi = 0x7FFFFFFF;
+            for (int c = 0, e = lane; e < E; ++c, e += 64) {
+                if (taken & (1u << c)) continue;
+                const float v = my[e];
+                if (bi == 0x7FFFFFFF || better(v, e, bv, bi)) {
+                    bv = v;
+                    bi = e;
+                }
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                const float ov = __shfl_xor(bv, off, 64);
+                const int oi = __shfl_xor(bi, off, 64);
+                if (oi != 0x7FFFFFFF && (bi == 0x7FFFFFFF || better(ov, oi, bv, bi))) {
+                    bv = ov;
+                    bi = oi;
+                }
+            }
+            sel_v[r] = bv;
+            sel_i[r] = bi;
+            if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
+        }
+    }
+    float outv[8];
+    if (do_softmax) {
+        double max_val = sel_v[0];
+#pragma unroll
+        for (int r = 1; r < 8; ++r)
+            if (r < K && sel_v[r] > max_val) max_val = sel_v[r];
+        double sum = 0.0;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            if (r < K) {
+                outv[r] = expf((float)((double)sel_v[r] - max_val));
+                sum += outv[r];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            if (r < K) outv[r] = (float)((double)outv[r] / sum);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) outv[r] = sel_v[r];
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        if (r < K && lane == r) {
+            topk_v[(size_t)t * K + r] = outv[r];
+            topk_i[(size_t)t * K + r] = sel_i[r];
+        }
+    }
+}
+
+// In-place softmax over the last dimension, one thread per row, the reference's order of
+// operations (src/run.cpp:321-339).
+__global__ void softmax_rows_kernel(float* __restrict__ x, int B, int size) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    float* r = x + (size_t)b * size;
+    double max_val = r[0];
+    for (int i = 1; i < size; ++i)
+        if (r[i] > max_val) max_val = r[i];
+    double sum = 0.0;
+    for (int i = 0; i < size; ++i) {
+        const float ex = expf((float)((double)r[i] - max_val));
+        r[i] = ex;
+        sum += ex;
+    }
+    for (int i = 0; i < size; ++i) r[i] = (float)((double)r[i] / sum);
+}
+
+// fp32 -> bf16 copy of the block input (operand of the expert GEMMs), 8 elements per thread.
+__global__ void convert_f32_bf16_kernel(const float* __restrict__ in, uint16_t* __restrict__ out, size_t n8) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    const float4 a = reinterpret_cast<const float4*>(in)[2 * i];
+    const float4 b = reinterpret_cast<const float4*>(in)[2 * i + 1];
+    uint4 o;
+    o.x = pack_bf16x2(a.x, a.y);
+    o.y = pack_bf16x2(a.z, a.w);
+    o.z = pack_bf16x2(b.x, b.y);
+    o.w = pack_bf16x2(b.z, b.w);
+    reinterpret_cast<uint4*>(out)[i] = o;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host launchers
+// ---------------------------------------------------------------------------------------------
+int router_segments(int T, int E, int H, bool strict) {
+    if (strict) return 1;
+    // enough (token tile, expert, segment) waves to cover the chip a few times over
+    const long long waves_one = (long long)ceil_div(T, 64) * E;
+    int S = 1;
+    while (S < 16 && waves_one * S < 4096 && H / (S * 2) >= 64) S *= 2;
+    return S;
+}
+
+size_t router_partial_bytes(int T, int E) { return (size_t)16 * T * E * sizeof(double); }
+
+int launch_router_partial(const float* x, const uint16_t* w, double* partial, int T, int H, int E, int S,
+                          hipStream_t stream) {
+    int seg_len = ceil_div(ceil_div(H, S), 8) * 8;
+    const long long waves1 = (long long)ceil_div(T, 64) * E * S;
+    // few waves: one expert per wave for parallelism; many: four per wave to reuse each LDS read
+    if (waves1 <= 8192) {
+        dim3 grid(ceil_div(T, 64), ceil_div(E, 4), S);
+        hipLaunchKernelGGL(router_partial_kernel<1>, grid, dim3(256), 0, stream, x, w, partial, T, H, E, seg_len);
+    } else {
+        dim3 grid(ceil_div(T, 64), ceil_div(E, 16), S);
+        hipLaunchKernelGGL(router_partial_kernel<4>, grid, dim3(256), 0, stream, x, w, partial, T, H, E, seg_len);
+    }
+    return launch_status();
+}
+
+int launch_router_finalize(const double* partial, int S, const float* scores_in, const uint16_t* bias,
+                           float* scores_out, float* topk_v, int* topk_i, int T, int E, int K, int do_topk,
+                           int do_softmax, hipStream_t stream) {
+    hipLaunchKernelGGL(router_finalize_kernel, dim3(ceil_div(T, 4)), dim3(256), (size_t)4 * E * sizeof(float),
+                       stream, partial, S, scores_in, bias, scores_out, topk_v, topk_i, T, E, K, do_topk,
+                       do_softmax);
+    return launch_status();
+}
+
+int launch_softmax_rows(float* x, int B, int size, hipStream_t stream) {
+    hipLaunchKernelGGL(softmax_rows_kernel, dim3(ceil_div(B, 256)), dim3(256), 0, stream, x, B, size);
+    return launch_status();
+}
+
+int launch_convert_f32_bf16(const float* in, uint16_t* out, size_t n, hipStream_t stream) {
+    const size_t n8 = n / 8;
+    hipLaunchKernelGGL(convert_f32_bf16_kernel, dim3((unsigned)ceil_div(n8, (size_t)256)), dim3(256), 0, stream,
+                       in, out, n8);
+    return launch_status();
+}
+
+}  // namespace moe
