@@ -62,7 +62,7 @@ int check_dims(int T, int H, int I, int E, int K) {
     if (H % 64 != 0 || I % 64 != 0) return MOE_ERR_SHAPE;
     if (K > E) return MOE_ERR_SHAPE;
     if (E > 1024 || K > 8) return MOE_ERR_LIMIT;
-    if ((long long)T * K > 0x7FFFFFFFll / 4) return MOE_ERR_LIMIT;
+    if (T > 65535) return MOE_ERR_LIMIT;  // one grid row per token in the combine kernel
     return MOE_OK;
 }
 
@@ -96,6 +96,7 @@ int moe_gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, cons
     if (!xout || !x_batch || !w || !bias) return MOE_ERR_NULL;
     if (N <= 0 || K <= 0 || M <= 0 || K % 8 != 0) return MOE_ERR_SHAPE;
     if (M > 1024) return MOE_ERR_LIMIT;
+    if (((uintptr_t)x_batch | (uintptr_t)w) & 15u) return MOE_ERR_ALIGN;
     const int S = router_segments(N, M, K, false);
     if (!scratch || ((uintptr_t)scratch & 7u) || scratch_bytes < (size_t)S * N * M * sizeof(double))
         return MOE_ERR_WORKSPACE;

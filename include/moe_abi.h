@@ -70,7 +70,8 @@ MOE_API const char* moe_error_string(int code);
  * Arithmetic follows the reference's CPU matmul (src/run.cpp:341-354): the product is an fp32
  * multiply of the fp32 activation with the widened bf16 weight, accumulated in fp64, rounded to
  * fp32, then the bias is added in fp32 (src/run.cpp:635-637).  Needs `scratch` of
- * moe_router_scratch_bytes(N, M) bytes (8-byte aligned).  M <= 1024, K % 4 == 0. */
+ * moe_router_scratch_bytes(N, M) bytes (8-byte aligned).  M <= 1024, K % 8 == 0; x_batch and w
+ * 16-byte aligned. */
 MOE_API size_t moe_router_scratch_bytes(int N, int M);
 MOE_API int moe_gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias,
                     int N, int K, int M, void* scratch, size_t scratch_bytes, moe_stream_t stream);
@@ -199,7 +200,7 @@ MOE_API int moe_mxfp4_tiled_to_bf16(const uint8_t* tiled_blocks, const uint8_t* 
  * ---------------------------------------------------------------------------------------- */
 typedef struct moe_block_params {
     uint32_t struct_bytes;   /* sizeof(moe_block_params), for forward compatibility */
-    int32_t n_tokens;        /* B */
+    int32_t n_tokens;        /* B <= 65535 */
     int32_t hidden_dim;      /* H, % 64 == 0 */
     int32_t intermediate_dim;/* I, % 64 == 0 */
     int32_t n_experts;       /* E <= 1024 */

@@ -57,7 +57,8 @@ def test_entries_reject_bad_arguments_without_a_device(pkg):
     assert L.moe_topk(1, 1, 1, 1, 4, 5, None) == -2
     assert L.moe_softmax(1, 4, 65, None) == -3
     assert L.moe_gemm_router(1, 1, 1, 1, 4, 2881, 32, 1, 1 << 30, None) == -2
-    assert L.moe_gemm_router(8, 8, 8, 8, 4, 2880, 32, None, 0, None) == -4
+    assert L.moe_gemm_router(16, 16, 16, 16, 4, 2880, 32, None, 0, None) == -4
+    assert L.moe_gemm_router(16, 8, 16, 16, 4, 2880, 32, 16, 1 << 30, None) == -6
     assert L.moe_bucket_by_expert(1, 1, 4, 4, 2000, 1, 1, 1, None, None) == -3
     assert L.moe_gather_rows(1, 1, 1, 4, 6, None) == -2
     assert L.moe_dequant_mxfp4(8, 8, 4, 8, None) == -6      # blocks not 16-byte aligned
