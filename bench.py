@@ -1,0 +1,177 @@
+"""Benchmark of the MoE expert block on one MI355X.
+
+A step is one pass of the whole block (router -> top-k -> softmax -> bucketing -> gate/up GEMM +
+SwiGLU -> down GEMM -> combine) over one batch of synthetic tokens already resident in HBM.
+Headline workload: the gpt-oss-20b-shaped block at 256-token decode with bf16 experts.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the gate/up GEMM, 2/3 of the
+weight bytes): algorithmic bytes of that launch / its average duration from HIP events recorded on
+the launch stream, against the 8 TB/s HBM peak.  `cpu_baseline` is the CPU oracle (the OpenMP
+restatement of the reference's CPU path) timed on the host cores on a bounded sample.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="decode256_bf16")
+    ap.add_argument("--also", default="decode256_mxfp4,prefill4096_mxfp4_zipf",
+                    help="comma-separated extra workloads reported under 'also' ('' for none)")
+    ap.add_argument("--cpu-tokens", type=int, default=256, help="tokens of the workload the CPU baseline runs")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--flags", type=int, default=0)
+    return ap.parse_args()
+
+
+def measure(pkg, wl, torch, shape, table, steps, warmup, flags=0):
+    """Returns a dict of measurements for one workload on cuda:0."""
+    dev = torch.device("cuda:0")
+    blk, raw = wl.make_device_layer(shape, table, dev)
+    x = wl.make_device_input(shape, table, dev)
+    T = shape.T
+    e_agg = torch.empty((T, shape.H), dtype=torch.float32, device=dev)
+    topk_i = torch.empty((T, shape.K), dtype=torch.int32, device=dev)
+    topk_v = torch.empty((T, shape.K), dtype=torch.float32, device=dev)
+    p = blk.params(x, e_agg, topk_i, topk_v, flags=flags)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    for _ in range(warmup):
+        blk.launch(p, stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        blk.launch(p, stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / steps
+
+    # second pass with HIP events at the stage boundaries (same stream)
+    timer = pkg.StageTimer()
+    stage_ms = [0.0] * len(pkg.STAGES)
+    for _ in range(steps):
+        timer.launch(p, stream)
+        for i, v in enumerate(timer.read()):
+            stage_ms[i] += v / steps
+    timer.close()
+
+    counts = torch.bincount(topk_i.flatten().long(), minlength=shape.E).cpu().numpy()
+    active = int((counts > 0).sum())
+    H, I = shape.H, shape.I
+    wpe = wl.weight_bytes_per_expert(shape)
+    w1_bytes = wpe * 2 // 3
+    w2_bytes = wpe - w1_bytes
+    bytes_mlp1 = active * (w1_bytes + 2 * I * 2) + T * H * 4
+    bytes_mlp2 = active * (w2_bytes + H * 2) + T * H * 4
+    flops_mlp1 = shape.K * T * 2 * (2 * I * H)
+    alg_bytes = wl.algorithmic_bytes(shape, active)
+    alg_flops = wl.algorithmic_flops(shape)
+    res = {
+        "workload": shape.name,
+        "ms_per_step": ms_per_step,
+        "tokens_per_s": T / (ms_per_step * 1e-3),
+        "stage_ms": dict(zip(pkg.STAGES, [round(v, 5) for v in stage_ms])),
+        "active_experts": active,
+        "rows_per_expert_min_max": [int(counts.min()), int(counts.max())],
+        "block_algorithmic_bytes": alg_bytes,
+        "block_hbm_frac": alg_bytes / (ms_per_step * 1e-3) / (HBM_PEAK_GBS * 1e9),
+        "block_mfma_frac": alg_flops / (ms_per_step * 1e-3) / (MFMA_BF16_PEAK_TFLOPS * 1e12),
+        "mlp1": {"bytes": bytes_mlp1, "flops": flops_mlp1, "ms": stage_ms[3]},
+        "mlp2": {"bytes": bytes_mlp2, "ms": stage_ms[4]},
+    }
+    del blk, raw, x
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline(ge, wl, shape, n_tokens):
+    """The CPU oracle on the first n_tokens of the workload, all host threads."""
+    sys.path.insert(0, os.path.join(ge.ROOT, "tests"))
+    import hostgen
+    oracle = ge.import_oracle()
+    hw = hostgen.host_layer(oracle, wl, shape)
+    x = hostgen.host_input(oracle, wl, shape)[:n_tokens]
+    hostgen.oracle_block(oracle, shape, hw, x[:2])  # warm the pages
+    t0 = time.perf_counter()
+    hostgen.oracle_block(oracle, shape, hw, x)
+    dt = time.perf_counter() - t0
+    return {"value": n_tokens / dt, "unit": "tokens/s", "cores": oracle.max_threads(), "kind": "port",
+            "sample": "%d tokens of %s through oracle/moe_oracle.c (fp32 weights, OpenMP over output rows), %.2f s"
+                      % (n_tokens, shape.name, dt)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X; --gpus %d is not supported (the MoE block is built for a single GPU: "
+              "no expert parallelism, no collectives)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import __graft_entry__ as ge
+    pkg = ge.import_package()
+    wl = importlib.import_module("gpt_oss_amd_amd.workloads")
+    oracle = ge.import_oracle()  # normal-quantile table of the synthetic generator + CPU baseline
+    table = oracle.normal_table()
+
+    shape = wl.WORKLOADS[args.workload]
+    head = measure(pkg, wl, torch, shape, table, args.steps, args.warmup, args.flags)
+    bound = "hbm" if shape.T <= 1024 else "mfma"
+    if bound == "hbm":
+        achieved = head["mlp1"]["bytes"] / (head["mlp1"]["ms"] * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "expert_stream_kernel (gate/up GEMM + SwiGLU)", "achieved": achieved,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None}
+    else:
+        achieved = head["mlp1"]["flops"] / (head["mlp1"]["ms"] * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": "gate/up GEMM + SwiGLU", "achieved": achieved,
+                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                    "traffic": None}
+
+    also = []
+    for name in [n for n in args.also.split(",") if n and n != args.workload]:
+        r = measure(pkg, wl, torch, wl.WORKLOADS[name], table, max(10, args.steps // 4), max(3, args.warmup // 4),
+                    args.flags)
+        also.append({k: r[k] for k in ("workload", "ms_per_step", "tokens_per_s", "block_hbm_frac", "block_mfma_frac",
+                                       "stage_ms", "rows_per_expert_min_max")})
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(ge, wl, shape, min(args.cpu_tokens, shape.T))
+
+    out = {
+        "metric": "MoE-block tokens/sec at 1 GPU; % HBM peak (decode), % bf16 MFMA peak (prefill)",
+        "value": head["tokens_per_s"],
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "%s: gpt-oss-20b-shaped MoE block, T=%d tokens, H=I=%d, E=%d, top-%d, %s experts"
+                               % (shape.name, shape.T, shape.H, shape.E, shape.K, shape.fmt),
+                   "tokens": shape.T, "active_experts": head["active_experts"]},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "block_hbm_frac": head["block_hbm_frac"],
+        "block_mfma_frac": head["block_mfma_frac"],
+        "stage_ms": head["stage_ms"],
+        "also": also,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -88,6 +88,10 @@ SIGNATURES = {
     "moe_mxfp4_tiled_to_bf16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "moe_block_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "moe_block_forward": (_i, [_c.POINTER(BlockParams), _vp]),
+    "moe_stage_timer_create": (_i, [_c.POINTER(_vp)]),
+    "moe_stage_timer_destroy": (None, [_vp]),
+    "moe_block_forward_timed": (_i, [_c.POINTER(BlockParams), _vp, _vp]),
+    "moe_stage_timer_read": (_i, [_vp, _c.POINTER(_f)]),
     "moe_synth_normal_f32": (_i, [_vp, _ll, _vp, _f, _u, _u, _vp]),
     "moe_synth_normal_bf16": (_i, [_vp, _ll, _vp, _f, _u, _u, _vp]),
     "moe_synth_bytes": (_i, [_vp, _ll, _u, _u, _vp]),
@@ -327,6 +331,33 @@ class MoeBlock:
         rc = _lib.moe_block_forward(ctypes.byref(p), stream)
         if rc:
             raise MoeError("moe_block_forward", rc)
+
+
+STAGES = ("router_partial", "router_finalize", "bucket", "mlp1_swiglu", "mlp2", "combine")
+
+
+class StageTimer:
+    """HIP-event timer for the six stages of moe_block_forward (moe_stage_timer of the C ABI)."""
+
+    def __init__(self):
+        self._h = _vp()
+        _check("moe_stage_timer_create", _lib.moe_stage_timer_create(ctypes.byref(self._h)))
+
+    def launch(self, p, stream):
+        _check("moe_block_forward_timed", _lib.moe_block_forward_timed(ctypes.byref(p), stream, self._h))
+
+    def read(self):
+        out = (_f * len(STAGES))()
+        _check("moe_stage_timer_read", _lib.moe_stage_timer_read(self._h, out))
+        return list(out)
+
+    def close(self):
+        if self._h:
+            _lib.moe_stage_timer_destroy(self._h)
+            self._h = _vp()
+
+    def __del__(self):
+        self.close()
 
 
 # ---- synthetic workloads (include/moe_synth.h) --------------------------------------------------

@@ -3,6 +3,9 @@
 #include "common.h"
 #include "kernels.h"
 
+#include <algorithm>
+#include <new>
+
 using namespace moe;
 
 namespace {
@@ -185,6 +188,7 @@ static int queue_gemm(int epi, int format, const int* work_queue, int work_start
     a.alpha = alpha;
     a.limit = limit;
     a.format = format;
+    a.waves_per_block = 4;
     return launch_expert_stream(a, epi, as_stream(stream));
 }
 
@@ -306,7 +310,11 @@ size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int intermediate_
     return BlockWorkspace(nullptr, n_tokens, hidden_dim, intermediate_dim, n_experts, experts_per_token).bytes;
 }
 
-int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
+struct moe_stage_timer {
+    hipEvent_t ev[MOE_N_STAGES + 1];
+};
+
+static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, moe_stage_timer* timer) {
     if (!p) return MOE_ERR_NULL;
     if (p->struct_bytes != sizeof(moe_block_params)) return MOE_ERR_FORMAT;
     const int T = p->n_tokens, H = p->hidden_dim, I = p->intermediate_dim, E = p->n_experts,
@@ -326,22 +334,31 @@ int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
     BlockWorkspace ws(p->workspace, T, H, I, E, K);
     if (p->workspace_bytes < ws.bytes) return MOE_ERR_WORKSPACE;
     hipStream_t stream = as_stream(stream_);
+    int stage = 0;
+    auto mark = [&]() -> int {
+        if (!timer) return MOE_OK;
+        return (int)hipEventRecord(timer->ev[stage++], stream);
+    };
+    if ((rc = mark())) return rc;
 
     // 1. router logits -> top-k -> softmax  (src/forward.cpp:318-327; src/run.cpp:630-642)
     const int S = router_segments(T, E, H, (p->flags & MOE_FLAG_ROUTER_STRICT_ORDER) != 0);
     rc = launch_router_partial(p->t, p->w_router, ws.router_partial, T, H, E, S, stream);
     if (rc) return rc;
+    if ((rc = mark())) return rc;
     rc = launch_router_finalize(ws.router_partial, S, nullptr, p->b_router, p->router_score, p->topk_v, p->topk_i, T, E,
                                 K, 1, 1, stream);
     if (rc) return rc;
     rc = launch_convert_f32_bf16(p->t, ws.t_bf16, (size_t)T * H, stream);
     if (rc) return rc;
+    if ((rc = mark())) return rc;
 
     // 2. bucketing + token-block map  (src/forward.cpp:329-376)
     TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, kStreamTileTokens, ws.max_tiles};
     rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat, ws.slot_of,
                        map, stream);
     if (rc) return rc;
+    if ((rc = mark())) return rc;
 
     // 3. gate/up GEMM + SwiGLU  (src/forward.cpp:474-479; src/run.cpp:657-689)
     ExpertGemmArgs g{};
@@ -355,6 +372,13 @@ int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
     g.limit = p->swiglu_limit;
     g.format = fmt;
 
+    // eight waves (256 weight rows) per block when that still yields enough blocks to fill the chip
+    const int est_tiles = std::max(ceil_div(T * K, kStreamTileTokens), std::min(E, T * K));
+    auto pick_waves = [&](int rows) { return ceil_div(rows / 32, 8) * est_tiles >= 512 ? 8 : 4; };
+    // measured on MI355X at decode shapes: bf16 weights stream fastest with uniform waves, MXFP4
+    // weights (four times the work per byte) with producer/consumer waves
+    auto pick_kernel = [&](int rows) { return fmt == MOE_WEIGHTS_BF16 ? pick_waves(rows) : 0; };
+
     ExpertGemmArgs a1 = g;
     a1.w = p->w_mlp1;
     a1.w_scales = static_cast<const uint8_t*>(p->w_mlp1_scales);
@@ -365,6 +389,7 @@ int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
     a1.rows = 2 * I;
     a1.K = H;
     a1.bias_expert_stride = 2LL * I;
+    a1.waves_per_block = pick_kernel(2 * I);
     if (fmt == MOE_WEIGHTS_BF16) {
         a1.w_expert_stride = 2LL * I * H;
     } else {
@@ -375,6 +400,7 @@ int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
     }
     rc = launch_expert_stream(a1, 0, stream);
     if (rc) return rc;
+    if ((rc = mark())) return rc;
 
     // 4. down GEMM  (src/forward.cpp:481-487; src/run.cpp:691-700)
     ExpertGemmArgs a2 = g;
@@ -387,6 +413,7 @@ int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
     a2.rows = H;
     a2.K = I;
     a2.bias_expert_stride = H;
+    a2.waves_per_block = pick_kernel(H);
     if (fmt == MOE_WEIGHTS_BF16) {
         a2.w_expert_stride = (long long)H * I;
     } else {
@@ -397,9 +424,48 @@ int moe_block_forward(const moe_block_params* p, moe_stream_t stream_) {
     }
     rc = launch_expert_stream(a2, 1, stream);
     if (rc) return rc;
+    if ((rc = mark())) return rc;
 
     // 5. weighted combine in ascending expert id (+ residual)  (src/run.cpp:702-712)
-    return launch_combine(ws.y_by_slot, ws.slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x, T, K, H, stream);
+    rc = launch_combine(ws.y_by_slot, ws.slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x, T, K, H, stream);
+    if (rc) return rc;
+    return mark();
+}
+
+int moe_block_forward(const moe_block_params* p, moe_stream_t stream) { return block_forward_impl(p, stream, nullptr); }
+
+int moe_block_forward_timed(const moe_block_params* p, moe_stream_t stream, moe_stage_timer* timer) {
+    if (!timer) return MOE_ERR_NULL;
+    return block_forward_impl(p, stream, timer);
+}
+
+int moe_stage_timer_create(moe_stage_timer** out) {
+    if (!out) return MOE_ERR_NULL;
+    moe_stage_timer* t = new (std::nothrow) moe_stage_timer();
+    if (!t) return (int)hipErrorOutOfMemory;
+    for (int i = 0; i <= MOE_N_STAGES; ++i) {
+        hipError_t e = hipEventCreate(&t->ev[i]);
+        if (e != hipSuccess) {
+            for (int j = 0; j < i; ++j) (void)hipEventDestroy(t->ev[j]);
+            delete t;
+            return (int)e;
+        }
+    }
+    *out = t;
+    return MOE_OK;
+}
+
+void moe_stage_timer_destroy(moe_stage_timer* t) {
+    if (!t) return;
+    for (int i = 0; i <= MOE_N_STAGES; ++i) (void)hipEventDestroy(t->ev[i]);
+    delete t;
+}
+
+int moe_stage_timer_read(moe_stage_timer* t, float* stage_ms) {
+    if (!t || !stage_ms) return MOE_ERR_NULL;
+    MOE_RETURN_IF_HIP(hipEventSynchronize(t->ev[MOE_N_STAGES]));
+    for (int i = 0; i < MOE_N_STAGES; ++i) MOE_RETURN_IF_HIP(hipEventElapsedTime(&stage_ms[i], t->ev[i], t->ev[i + 1]));
+    return MOE_OK;
 }
 
 // ---- synthetic workloads ----------------------------------------------------------------------

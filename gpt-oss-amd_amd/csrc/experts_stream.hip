@@ -1,21 +1,23 @@
 // Weight-streaming expert GEMM for decode-sized buckets (tens of rows per expert).
 //
 // Every weight byte is loaded from HBM exactly once per token block, straight into the MFMA
-// A-operand registers with 128-bit loads (no LDS: a weight element is used by one wave only);
-// the few activation rows of the bucket are the B operand, read from the L2-resident bf16 copy.
-// fp32 accumulation in v_mfma_f32_16x16x32_bf16.  Replaces moe_mlp1_swiglu_mfma_kernel
-// (src/hip/moe.hip:9-235) and moe_mlp2_scatter_mfma_kernel (src/hip/moe.hip:261-512) for small
-// buckets; the arithmetic contract is the CPU path's (src/run.cpp:657-705): y = W x + b, SwiGLU on
-// interleaved gate/up rows, down projection.
+// A-operand registers with 128-bit loads (no LDS for weights: a weight element is used by one wave
+// only).  The bucket's activation rows are the B operand; the four waves of a block share them
+// through LDS, staged 128 contraction elements at a time in MFMA operand order (one contiguous
+// KiB per k-step and token tile, so the 128-bit LDS reads are conflict-free), double-buffered so
+// one barrier per stage suffices.  fp32 accumulation in v_mfma_f32_16x16x32_bf16.
+// Replaces moe_mlp1_swiglu_mfma_kernel (src/hip/moe.hip:9-235) and moe_mlp2_scatter_mfma_kernel
+// (src/hip/moe.hip:261-512) for small buckets; the arithmetic contract is the CPU path's
+// (src/run.cpp:657-705): y = W x + b, SwiGLU on interleaved gate/up rows, down projection.
 //
-// Work split: block (x = row unit, y = token block).  A block has 4 waves; each wave owns R MFMA
-// row tiles (16R weight rows) over the whole contraction length and up to NT*16 tokens.
+// Work split: block (x = group of row units, y = token block).  A block has 4 waves; each wave
+// owns R MFMA row tiles (16R weight rows) over the whole contraction length and up to NT*16 tokens.
 // The contraction index is a dummy index, so lanes are free to pick which k each of their eight
-// operand elements stands for as long as A and B agree:
-//   bf16  : per 64-element chunk, lane group g = lane/16 takes elements [16g, 16g+16): two adjacent
-//           128-bit loads per row, a whole 128-byte line per row per chunk;
-//   MXFP4 : per 128-element chunk, lane group g takes MX block g of the chunk (32 elements, one
-//           128-bit load + one scale byte), dequantised in registers to four A operands.
+// operand elements stands for as long as A and B agree.  Inside a stage of 128 elements, k-step j
+// (0..3) and lane group g = lane/16 take
+//   bf16  : elements 32j + 8g .. +8   (one 128-bit load per row tile and k-step)
+//   MXFP4 : elements 32g + 8j .. +8   (lane group g owns MX block g of the stage: one 128-bit load
+//           + one scale byte per row tile and stage, dequantised in registers to four A operands)
 #include "common.h"
 #include "kernels.h"
 
@@ -26,187 +28,27 @@ namespace {
 constexpr int FMT_BF16 = MOE_WEIGHTS_BF16;
 constexpr int FMT_MXFP4 = MOE_WEIGHTS_MXFP4_TILED;
 
-template <int FMT>
-struct ChunkTraits;
-template <>
-struct ChunkTraits<FMT_BF16> {
-    static constexpr int kElems = 64;   // contraction elements per chunk
-    static constexpr int kSteps = 2;    // MFMA k-steps per chunk
-    static constexpr int kADwords = 8;  // raw A dwords per lane per row tile per chunk
-};
-template <>
-struct ChunkTraits<FMT_MXFP4> {
-    static constexpr int kElems = 128;
-    static constexpr int kSteps = 4;
-    static constexpr int kADwords = 4;
-};
-
 // Epilogues: the fused block keeps bf16 SwiGLU outputs and fp32 per-slot rows; the entries that
 // keep the reference's data flow write fp32 SwiGLU outputs and scatter with atomics.
 enum { EPI_SWIGLU_BF16 = 0, EPI_ROWS_F32 = 1, EPI_SWIGLU_F32 = 2, EPI_SCATTER = 3 };
 
-template <int FMT, int R, int NT>
-struct Frags {
-    u32x4 a[R][ChunkTraits<FMT>::kADwords / 4];  // raw weight data
-    u32x4 b[NT][ChunkTraits<FMT>::kSteps];       // bf16 activations
-};
+constexpr int kStageSteps = 4;                                  // MFMA k-steps per LDS stage
+constexpr int kStageElems = 32 * kStageSteps;                   // 128 contraction elements
+constexpr int kNTMax = 4;                                       // token tiles (of 16) per block
+constexpr int kLdsStageBytes = kStageSteps * kNTMax * 1024;     // 16 KiB, two of them per block
 
 MOE_DEVICE u32x4 pack_f32x8_to_bf16x8(const float4& lo, const float4& hi) {
     return u32x4{pack_bf16x2(lo.x, lo.y), pack_bf16x2(lo.z, lo.w), pack_bf16x2(hi.x, hi.y), pack_bf16x2(hi.z, hi.w)};
 }
 
-// One (row unit, token block) of one expert.  ACT_F32: activations are fp32 rows indexed by slot
-// (the reference's x_by_expert / gate_by_expert buffers) and are rounded to bf16 on load.
-template <int FMT, int R, int NT, int EPI, bool ACT_F32>
-MOE_DEVICE void stream_body(const ExpertGemmArgs& a, int e, int row0, int nrows, int unit) {
-    using CT = ChunkTraits<FMT>;
-    constexpr int kUnitsPerGroup = 4 / R;
+// Epilogue shared by the expert kernels: lane (q,g) of the 16x16 accumulator layout holds token
+// t*16+q and weight rows group*64 + g*16 + (r0+r)*4 + j (j = 0..3) for its R row tiles.
+template <int R, int NT, int EPI>
+MOE_DEVICE void stream_epilogue(const ExpertGemmArgs& a, const f32x4 (&acc)[R][NT], int e, int row0, int nrows,
+                                int group, int r0) {
     const int lane = threadIdx.x & 63;
     const int q = lane & 15;
     const int g = lane >> 4;
-    const int group = unit / kUnitsPerGroup;
-    const int r0 = (unit % kUnitsPerGroup) * R;
-    const int K = a.K;
-
-    // ---- operand addressing ----
-    const uint8_t* a_ptr[R];
-    const uint8_t* s_ptr[R];
-    if constexpr (FMT == FMT_BF16) {
-        const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int row = group * 64 + tile_row_in_group(r0 + r, q);
-            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 16 * g);
-            s_ptr[r] = nullptr;
-        }
-    } else {
-        const int G = K / 32;
-        const size_t tile_bytes = (size_t)G * 256;
-        const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
-        const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
-        const uint8_t* sbase = a.w_scales + (size_t)e * a.s_expert_stride;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const size_t tile = (size_t)group * 4 + (r0 + r);
-            a_ptr[r] = wbase + tile * tile_bytes + (size_t)lane * 16;
-            s_ptr[r] = sbase + tile * stile_bytes + (size_t)lane * 4;
-        }
-    }
-    const uint8_t* b_ptr[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        const int idx = min(t * 16 + q, nrows - 1);
-        if constexpr (ACT_F32) {
-            b_ptr[t] = reinterpret_cast<const uint8_t*>(a.act_f32 + (size_t)(row0 + idx) * K) +
-                       (FMT == FMT_BF16 ? 64 * g : 128 * g);
-        } else {
-            const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
-            b_ptr[t] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K) +
-                       (FMT == FMT_BF16 ? 32 * g : 64 * g);
-        }
-    }
-
-    f32x4 acc[R][NT];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    const int n_chunks = ceil_div(K, CT::kElems);
-    const int rem_groups = (FMT == FMT_MXFP4) ? ((K / 32) & 3) : 0;  // MX blocks in a ragged last chunk
-
-    uint32_t scale_word[R];  // four scale bytes, one per chunk, reloaded every fourth chunk
-
-    auto load_chunk = [&](Frags<FMT, R, NT>& f, int c) {
-        if constexpr (FMT == FMT_BF16) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const u32x4* p = reinterpret_cast<const u32x4*>(a_ptr[r] + (size_t)c * 128);
-                f.a[r][0] = p[0];
-                f.a[r][1] = p[1];
-            }
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                if constexpr (ACT_F32) {
-                    const float4* p = reinterpret_cast<const float4*>(b_ptr[t] + (size_t)c * 256);
-                    f.b[t][0] = pack_f32x8_to_bf16x8(p[0], p[1]);
-                    f.b[t][1] = pack_f32x8_to_bf16x8(p[2], p[3]);
-                } else {
-                    const u32x4* p = reinterpret_cast<const u32x4*>(b_ptr[t] + (size_t)c * 128);
-                    f.b[t][0] = p[0];
-                    f.b[t][1] = p[1];
-                }
-            }
-        } else {
-            const bool live = !(rem_groups != 0 && c == n_chunks - 1 && g >= rem_groups);
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                f.a[r][0] = u32x4{0u, 0u, 0u, 0u};
-                if (live) f.a[r][0] = *reinterpret_cast<const u32x4*>(a_ptr[r] + (size_t)c * 1024);
-            }
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    f.b[t][s] = u32x4{0u, 0u, 0u, 0u};
-                    if (live) {
-                        if constexpr (ACT_F32) {
-                            const float4* p = reinterpret_cast<const float4*>(b_ptr[t] + (size_t)c * 512);
-                            f.b[t][s] = pack_f32x8_to_bf16x8(p[2 * s], p[2 * s + 1]);
-                        } else {
-                            const u32x4* p = reinterpret_cast<const u32x4*>(b_ptr[t] + (size_t)c * 256);
-                            f.b[t][s] = p[s];
-                        }
-                    }
-                }
-            }
-        }
-    };
-
-    auto compute_chunk = [&](const Frags<FMT, R, NT>& f, int c) {
-        if constexpr (FMT == FMT_BF16) {
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(f.a[r][s], f.b[t][s], acc[r][t]);
-        } else {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const float sc = mxfp4_scale_to_f32((scale_word[r] >> (8 * (c & 3))) & 0xFFu);
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    uint32_t d[4];
-                    mxfp4_dword_to_bf16x8(f.a[r][0][s], sc, d);
-                    const u32x4 av = {d[0], d[1], d[2], d[3]};
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, f.b[t][s], acc[r][t]);
-                }
-            }
-        }
-    };
-
-    auto load_scales = [&](int c) {
-        if constexpr (FMT == FMT_MXFP4) {
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                scale_word[r] = *reinterpret_cast<const uint32_t*>(s_ptr[r] + (size_t)(c >> 2) * 256);
-        }
-    };
-
-    Frags<FMT, R, NT> f0, f1;
-    load_scales(0);
-    load_chunk(f0, 0);
-    for (int c = 0; c < n_chunks; c += 2) {
-        if (c + 1 < n_chunks) load_chunk(f1, c + 1);
-        compute_chunk(f0, c);
-        if (c + 2 < n_chunks) load_chunk(f0, c + 2);
-        if (c + 1 < n_chunks) compute_chunk(f1, c + 1);
-        if (((c + 2) & 3) == 0 && c + 2 < n_chunks) load_scales(c + 2);
-    }
-
-    // ---- epilogue: lane (q,g) holds token t*16+q, weight rows group*64 + g*16 + (r0+r)*4 + j ----
     const int row_base = group * 64 + g * 16 + r0 * 4;
     const uint16_t* bias = a.bias + (size_t)e * a.bias_expert_stride + row_base;
     float bv[R][4];
@@ -270,54 +112,522 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, int e, int row0, int nrows,
     }
 }
 
-template <int FMT, int R, int EPI, bool ACT_F32>
-MOE_DEVICE void stream_dispatch(const ExpertGemmArgs& a, int e, int row0, int nrows, int unit) {
-    const int nt = (nrows + 15) >> 4;
-    if (nt == 4) {
-        stream_body<FMT, R, 4, EPI, ACT_F32>(a, e, row0, nrows, unit);
-    } else if (nt == 3) {
-        stream_body<FMT, R, 3, EPI, ACT_F32>(a, e, row0, nrows, unit);
-    } else if (nt == 2) {
-        stream_body<FMT, R, 2, EPI, ACT_F32>(a, e, row0, nrows, unit);
-    } else if (nt == 1) {
-        stream_body<FMT, R, 1, EPI, ACT_F32>(a, e, row0, nrows, unit);
+// One (row unit, token block) of one expert.  ACT_F32: activations are fp32 rows indexed by slot
+// (the reference's x_by_expert / gate_by_expert buffers) and are rounded to bf16 while staged.
+// `active` is false for the waves of a ragged last block that own no rows: they still stage
+// activations and take part in every barrier.
+template <int FMT, int R, int NT, int EPI, bool ACT_F32, int WAVES>
+MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit,
+                            bool active) {
+    static_assert(WAVES == 4 || WAVES == 8, "a block has 4 or 8 waves");
+    constexpr int kStagers = WAVES / 4;                       // waves that stage the same k-step
+    constexpr int TS = (NT + kStagers - 1) / kStagers;        // token tiles staged per wave
+    constexpr int kUnitsPerGroup = 4 / R;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane & 15;
+    const int g = lane >> 4;
+    const int group = unit / kUnitsPerGroup;
+    const int r0 = (unit % kUnitsPerGroup) * R;
+    const int K = a.K;
+    const int n_stages = ceil_div(K, kStageElems);
+
+    // ---- A operand addressing ----
+    const uint8_t* a_ptr[R];
+    const uint8_t* s_ptr[R];
+    if constexpr (FMT == FMT_BF16) {
+        const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int row = active ? group * 64 + tile_row_in_group(r0 + r, q) : 0;
+            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 8 * g);
+            s_ptr[r] = nullptr;
+        }
+    } else {
+        const int G = K / 32;
+        const size_t tile_bytes = (size_t)G * 256;
+        const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
+        const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
+        const uint8_t* sbase = a.w_scales + (size_t)e * a.s_expert_stride;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const size_t tile = active ? (size_t)group * 4 + (r0 + r) : 0;
+            a_ptr[r] = wbase + tile * tile_bytes + (size_t)lane * 16;
+            s_ptr[r] = sbase + tile * stile_bytes + (size_t)lane * 4;
+        }
+    }
+
+    // ---- B staging: wave w stages k-step w%4 of every stage, for token tiles w/4, w/4 + WAVES/4, ...
+    // (a tile index past NT-1 stages a clamped copy into an LDS slot nobody reads) ----
+    const int step_w = wave & 3;
+    const int half_w = wave >> 2;
+    // element offset inside an activation row of this lane's eight elements at stage 0
+    const int k_lane = (FMT == FMT_BF16) ? (32 * step_w + 8 * g) : (32 * g + 8 * step_w);
+    const uint8_t* b_src[TS];
+#pragma unroll
+    for (int i = 0; i < TS; ++i) {
+        const int t = half_w + kStagers * i;
+        const int idx = min(t * 16 + q, nrows - 1);
+        if constexpr (ACT_F32) {
+            b_src[i] = reinterpret_cast<const uint8_t*>(a.act_f32 + (size_t)(row0 + idx) * K + k_lane);
+        } else {
+            const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
+            b_src[i] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K + k_lane);
+        }
+    }
+    uint8_t* const lds_wr = lds + (size_t)(step_w * kNTMax + half_w) * 1024 + (size_t)lane * 16;
+    const uint8_t* const lds_rd = lds + (size_t)lane * 16;
+
+    // Everything inside the stage loops is branch-free (clamped addresses + selects instead of
+    // guards), so the compiler can count outstanding loads exactly and keep the prefetches in flight.
+    u32x4 stg[TS];
+    auto stage_load = [&](int s) {
+        // s may point past the last stage (prefetch of a stage that does not exist): stage zeros
+        const bool live = (s * kStageElems + k_lane) < K;  // false in a ragged or non-existent stage
+        const size_t off = live ? (size_t)s * kStageElems : 0;
+#pragma unroll
+        for (int t = 0; t < TS; ++t) {
+            u32x4 v;
+            if constexpr (ACT_F32) {
+                const float4* p = reinterpret_cast<const float4*>(b_src[t] + off * 4 - (live ? 0 : k_lane * 4));
+                v = pack_f32x8_to_bf16x8(p[0], p[1]);
+            } else {
+                v = *reinterpret_cast<const u32x4*>(b_src[t] + off * 2 - (live ? 0 : k_lane * 2));
+            }
+            stg[t] = live ? v : u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+    auto stage_store = [&](int buf) {
+#pragma unroll
+        for (int t = 0; t < TS; ++t)
+            *reinterpret_cast<u32x4*>(lds_wr + (size_t)buf * kLdsStageBytes + t * kStagers * 1024) = stg[t];
+    };
+    auto b_frag = [&](int buf, int j, int t) {
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)buf * kLdsStageBytes + (j * kNTMax + t) * 1024);
+    };
+
+    if (!active) {
+        // no rows to compute: keep the block's staging and barrier sequence going
+        const int n_iter = (FMT == FMT_BF16) ? n_stages : ceil_div(n_stages, 4) * 4;
+        stage_load(0);
+        stage_store(0);
+        __syncthreads();
+        for (int s = 0; s < n_iter; ++s) {
+            stage_load(s + 1);
+            stage_store((s & 1) ^ 1);
+            __syncthreads();
+        }
+        return;
+    }
+
+    f32x4 acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if constexpr (FMT == FMT_BF16) {
+        // A ring of four k-steps, loads issued three steps ahead of their use
+        const int n_steps = K / 32;
+        const int n_full = K / kStageElems;  // stages with all four k-steps
+        u32x4 ar[4][R];
+        auto load_a = [&](int slot, int n) {
+            const size_t off = (size_t)min(n, n_steps - 1) * 64;  // past the end: reload the last step
+#pragma unroll
+            for (int r = 0; r < R; ++r) ar[slot][r] = *reinterpret_cast<const u32x4*>(a_ptr[r] + off);
+        };
+        auto step = [&](int buf, int j) {
+            u32x4 b[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) b[t] = b_frag(buf, j, t);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(ar[j][r], b[t], acc[r][t]);
+        };
+        stage_load(0);
+        load_a(0, 0);
+        load_a(1, 1);
+        load_a(2, 2);
+        stage_store(0);
+        __syncthreads();
+        for (int s = 0; s < n_full; ++s) {
+            const int buf = s & 1;
+            stage_load(s + 1);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                load_a((j + 3) & 3, 4 * s + j + 3);
+                step(buf, j);
+            }
+            stage_store(buf ^ 1);
+            __syncthreads();
+        }
+        if (n_full < n_stages) {  // ragged last stage: K % 128 in {32, 64, 96}
+            const int buf = n_full & 1;
+            const int left = n_steps - 4 * n_full;
+            step(buf, 0);
+            if (left > 1) step(buf, 1);
+            if (left > 2) step(buf, 2);
+            __syncthreads();
+        }
+    } else {
+        // A ring of four stages (one 128-bit load per row tile and stage), loads issued three stages
+        // ahead of their use; one scale word per row tile covers four stages and is fetched one
+        // quad ahead.  The stage count is padded to a multiple of four with all-zero stages (zero
+        // weights against zero activations) to keep the loop uniform.
+        constexpr int D = 4;
+        const int rem_groups = (K / 32) & 3;  // MX blocks in a ragged last stage (0 = none)
+        const int n_quads = ceil_div(n_stages, 4);
+        u32x4 araw[D][R];
+        uint32_t sw_cur[R], sw_nxt[R];
+        auto load_a = [&](int slot, int s) {
+            const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
+            // a dead lane group re-reads a block that exists and drops it
+            const size_t off = live ? (size_t)s * 1024 : 0;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[r] + off);
+                araw[slot][r] = live ? v : u32x4{0u, 0u, 0u, 0u};
+            }
+        };
+        auto load_scales = [&](uint32_t (&dst)[R], int quad) {
+            const size_t off = (size_t)min(quad, n_quads - 1) * 256;
+#pragma unroll
+            for (int r = 0; r < R; ++r) dst[r] = *reinterpret_cast<const uint32_t*>(s_ptr[r] + off);
+        };
+        auto do_stage = [&](int slot, int s) {
+            const int buf = s & 1;
+            stage_load(s + 1);
+            load_a((slot + D - 1) % D, s + D - 1);
+            float sc[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32((sw_cur[r] >> (8 * slot)) & 0xFFu);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                u32x4 b[NT];
+#pragma unroll
+                for (int t = 0; t < NT; ++t) b[t] = b_frag(buf, j, t);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    uint32_t d[4];
+                    mxfp4_dword_to_bf16x8(araw[slot][r][j], sc[r], d);
+                    const u32x4 av = {d[0], d[1], d[2], d[3]};
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
+                }
+            }
+            stage_store(buf ^ 1);
+            __syncthreads();
+        };
+        stage_load(0);
+        load_scales(sw_cur, 0);
+#pragma unroll
+        for (int i = 0; i < D - 1; ++i) load_a(i, i);
+        stage_store(0);
+        __syncthreads();
+        for (int qd = 0; qd < n_quads; ++qd) {
+            load_scales(sw_nxt, qd + 1);
+#pragma unroll
+            for (int i = 0; i < D; ++i) do_stage(i, 4 * qd + i);
+#pragma unroll
+            for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
+        }
+    }
+
+    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Warp-specialised variant used by the fused block: a block has ten consumer waves (R = 2 row
+// tiles each, 320 weight rows per block) and two producer waves.  Producers move the bucket's
+// activation rows global -> LDS with direct-to-LDS 128-bit loads (no registers, a ring of four
+// 16 KiB stage slots, three stages ahead of the consumers); consumers only have weight loads in
+// their memory queue, eight units (bf16: k-steps, MXFP4: stages) ahead of their use.  One barrier
+// per stage; every wave of the block executes exactly 1 + n_pad barriers.
+// Positions of the contraction range that do not exist (ragged last stage, padding stages) carry
+// a weight operand of exact zeros; the activation operand there is a clamped re-read of real data.
+// ---------------------------------------------------------------------------------------------
+constexpr int kWsConsumers = 10;
+constexpr int kWsProducers = 2;
+constexpr int kWsThreads = (kWsConsumers + kWsProducers) * 64;
+constexpr int kWsRing = 4;
+
+template <int N>
+MOE_DEVICE void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+MOE_DEVICE void dma16(const void* gsrc, uint8_t* lds_dst_wave_uniform) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 16, 0, 0);
+}
+
+template <int FMT>
+MOE_DEVICE int ws_padded_stages(int K) {
+    const int n_stages = ceil_div(K, kStageElems);
+    return (FMT == FMT_BF16) ? ceil_div(n_stages, 2) * 2 : ceil_div(n_stages, 6) * 6;
+}
+
+template <int FMT, int NT>
+MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int nrows, int p) {
+    constexpr int Q = 2 * NT;  // direct-to-LDS loads per stage issued by this wave
+    const int lane = threadIdx.x & 63;
+    const int q = lane & 15;
+    const int g = lane >> 4;
+    const int K = a.K;
+    const int n_pad = ws_padded_stages<FMT>(K);
+    const uint8_t* row[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int idx = min(t * 16 + q, nrows - 1);
+        const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
+        row[t] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
+    }
+    auto issue = [&](int s) {
+        uint8_t* slot = lds + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes;
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = 2 * p + jj;
+            const int k = (FMT == FMT_BF16) ? (s * kStageElems + 32 * j + 8 * g) : (s * kStageElems + 32 * g + 8 * j);
+            const size_t off = (k < K) ? (size_t)k * 2 : 0;  // a position past the row re-reads its start
+#pragma unroll
+            for (int t = 0; t < NT; ++t) dma16(row[t] + off, slot + (j * kNTMax + t) * 1024);
+        }
+    };
+    issue(0);
+    issue(1);
+    issue(2);
+    wait_vmcnt<2 * Q>();  // stage 0 has landed
+    __syncthreads();
+    for (int i = 0; i < n_pad; ++i) {
+        issue(i + 3);
+        wait_vmcnt<2 * Q>();  // stage i+1 has landed
+        __syncthreads();
+    }
+    wait_vmcnt<0>();  // nothing may still be writing this block's LDS when the wave ends
+}
+
+template <int FMT, int NT, int EPI>
+MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, int row0, int nrows, int unit,
+                            bool active) {
+    constexpr int R = 2;
+    const int lane = threadIdx.x & 63;
+    const int g = lane >> 4;
+    const int q = lane & 15;
+    const int K = a.K;
+    const int n_stages = ceil_div(K, kStageElems);
+    const int n_pad = ws_padded_stages<FMT>(K);
+    if (!active) {
+        for (int i = 0; i <= n_pad; ++i) __syncthreads();
+        return;
+    }
+    const int group = unit >> 1;
+    const int r0 = (unit & 1) * R;
+    const uint8_t* const lds_rd = lds + (size_t)lane * 16;
+    auto b_frag = [&](int s, int j, int t) {
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes +
+                                               (j * kNTMax + t) * 1024);
+    };
+    f32x4 acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if constexpr (FMT == FMT_BF16) {
+        constexpr int D = 8;  // ring of k-steps
+        const int n_steps = K / 32;
+        const uint8_t* a_ptr[R];
+        const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int row = group * 64 + tile_row_in_group(r0 + r, q);
+            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 8 * g);
+        }
+        u32x4 ar[D][R];
+        auto load_a = [&](int slot, int n) {
+            const bool live = n < n_steps;
+            const size_t off = live ? (size_t)n * 64 : 0;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[r] + off);
+                ar[slot][r] = live ? v : u32x4{0u, 0u, 0u, 0u};
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < D - 1; ++i) load_a(i, i);
+        __syncthreads();
+        for (int s0 = 0; s0 < n_pad; s0 += 2) {
+#pragma unroll
+            for (int ss = 0; ss < 2; ++ss) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int u = 4 * ss + j;
+                    load_a((u + D - 1) % D, 4 * (s0 + ss) + j + D - 1);
+                    u32x4 b[NT];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) b[t] = b_frag(s0 + ss, j, t);
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(ar[u][r], b[t], acc[r][t]);
+                }
+                __syncthreads();
+            }
+        }
+    } else {
+        constexpr int D = 6;  // ring of stages: one 128-bit load + one scale byte per row tile and stage
+        const int G = K / 32;
+        const int rem_groups = G & 3;  // MX blocks in a ragged last stage (0 = none)
+        const size_t tile_bytes = (size_t)G * 256;
+        const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
+        const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
+        const uint8_t* sbase = a.w_scales + (size_t)e * a.s_expert_stride;
+        const uint8_t* a_ptr[R];
+        const uint8_t* s_ptr[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const size_t tile = (size_t)group * 4 + (r0 + r);
+            a_ptr[r] = wbase + tile * tile_bytes + (size_t)lane * 16;
+            s_ptr[r] = sbase + tile * stile_bytes + (size_t)lane * 4;
+        }
+        u32x4 araw[D][R];
+        uint32_t sbyte[D][R];
+        auto load_a = [&](int slot, int s) {
+            const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
+            const int sc = live ? s : 0;  // a dead lane group re-reads a block that exists and drops it
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[r] + (size_t)sc * 1024);
+                araw[slot][r] = live ? v : u32x4{0u, 0u, 0u, 0u};
+                sbyte[slot][r] = *(s_ptr[r] + (size_t)(sc >> 2) * 256 + (sc & 3));
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < D - 1; ++i) load_a(i, i);
+        __syncthreads();
+        for (int s0 = 0; s0 < n_pad; s0 += D) {
+#pragma unroll
+            for (int u = 0; u < D; ++u) {
+                const int s = s0 + u;
+                load_a((u + D - 1) % D, s + D - 1);
+                float sc[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32(sbyte[u][r]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    u32x4 b[NT];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) b[t] = b_frag(s, j, t);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        uint32_t d[4];
+                        mxfp4_dword_to_bf16x8(araw[u][r][j], sc[r], d);
+                        const u32x4 av = {d[0], d[1], d[2], d[3]};
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0);
+}
+
+// grid = (ceil(row units / 10), max_tiles), block = 768 (waves 0-9 consume, 10-11 produce); three
+// waves per SIMD, i.e. one block per CU with up to 168 registers per lane.
+template <int FMT, int EPI>
+__global__ __launch_bounds__(kWsThreads, 3) void expert_stream_ws_kernel(ExpertGemmArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kWsRing * kLdsStageBytes];
+    const int tile = blockIdx.y;
+    if (tile >= *a.n_tiles) return;  // block-uniform
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int e = a.tile_expert[tile];
+    const int row0 = a.tile_row0[tile];
+    const int nrows = a.tile_rows[tile];
+    const int nt = (nrows + 15) >> 4;  // block-uniform
+    if (wave >= kWsConsumers) {
+        const int p = wave - kWsConsumers;
+        if (nt == 4) ws_producer<FMT, 4>(a, lds, row0, nrows, p);
+        else if (nt == 3) ws_producer<FMT, 3>(a, lds, row0, nrows, p);
+        else if (nt == 2) ws_producer<FMT, 2>(a, lds, row0, nrows, p);
+        else ws_producer<FMT, 1>(a, lds, row0, nrows, p);
+    } else {
+        const int unit = blockIdx.x * kWsConsumers + wave;
+        const bool active = unit < a.rows / 32;
+        if (nt == 4) ws_consumer<FMT, 4, EPI>(a, lds, e, row0, nrows, unit, active);
+        else if (nt == 3) ws_consumer<FMT, 3, EPI>(a, lds, e, row0, nrows, unit, active);
+        else if (nt == 2) ws_consumer<FMT, 2, EPI>(a, lds, e, row0, nrows, unit, active);
+        else ws_consumer<FMT, 1, EPI>(a, lds, e, row0, nrows, unit, active);
     }
 }
 
-// Token blocks from the bucketing kernel's tile map.  grid = (row units / 4, max_tiles).
-template <int FMT, int R, int EPI>
-__global__ __launch_bounds__(256) void expert_stream_kernel(ExpertGemmArgs a) {
+template <int FMT, int R, int EPI, bool ACT_F32, int WAVES>
+MOE_DEVICE void stream_dispatch(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit,
+                                bool active) {
+    const int nt = (nrows + 15) >> 4;  // block-uniform
+    if (nt == 4) {
+        stream_body<FMT, R, 4, EPI, ACT_F32, WAVES>(a, lds, e, row0, nrows, unit, active);
+    } else if (nt == 3) {
+        stream_body<FMT, R, 3, EPI, ACT_F32, WAVES>(a, lds, e, row0, nrows, unit, active);
+    } else if (nt == 2) {
+        stream_body<FMT, R, 2, EPI, ACT_F32, WAVES>(a, lds, e, row0, nrows, unit, active);
+    } else if (nt == 1) {
+        stream_body<FMT, R, 1, EPI, ACT_F32, WAVES>(a, lds, e, row0, nrows, unit, active);
+    }
+}
+
+// Token blocks from the bucketing kernel's tile map.  grid = (ceil(row units / WAVES), max_tiles).
+template <int FMT, int R, int EPI, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 4) void expert_stream_kernel(ExpertGemmArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kLdsStageBytes];
     const int tile = blockIdx.y;
-    if (tile >= *a.n_tiles) return;
+    if (tile >= *a.n_tiles) return;  // block-uniform
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * 4 + wave;
-    if (unit >= (a.rows / 64) * (4 / R)) return;
-    stream_dispatch<FMT, R, EPI, false>(a, a.tile_expert[tile], a.tile_row0[tile], a.tile_rows[tile], unit);
+    const int unit = blockIdx.x * WAVES + wave;
+    const bool active = unit < (a.rows / 64) * (4 / R);
+    stream_dispatch<FMT, R, EPI, false, WAVES>(a, lds, a.tile_expert[tile], a.tile_row0[tile], a.tile_rows[tile],
+                                               unit, active);
 }
 
 // Token blocks from a queue of (expert, row_offset, row_count) triples (entry format of
-// src/hip/scheduler.hip:163-166).  grid = (row units / 4, token blocks per entry, entries).
+// src/hip/scheduler.hip:163-166).  grid = (ceil(row units / 4), token blocks per entry, entries).
 template <int FMT, int R, int EPI>
 __global__ __launch_bounds__(256) void expert_stream_queue_kernel(ExpertGemmArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kLdsStageBytes];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int unit = blockIdx.x * 4 + wave;
-    if (unit >= (a.rows / 64) * (4 / R)) return;
+    const bool active = unit < (a.rows / 64) * (4 / R);
     const int* entry = a.work_queue + 3 * (a.work_start + blockIdx.z);
     const int e = entry[0], off = entry[1], n = entry[2];
-    for (int tb = blockIdx.y; tb * 64 < n; tb += gridDim.y)
-        stream_dispatch<FMT, R, EPI, true>(a, e, off + tb * 64, min(64, n - tb * 64), unit);
+    for (int tb = blockIdx.y; tb * 64 < n; tb += gridDim.y) {
+        stream_dispatch<FMT, R, EPI, true, 4>(a, lds, e, off + tb * 64, min(64, n - tb * 64), unit, active);
+        __syncthreads();  // the next token block restages both LDS buffers
+    }
 }
 
-template <int FMT, int R, int EPI>
+template <int FMT, int EPI>
 int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
+    constexpr int R = 2;
     const int units = (a.rows / 64) * (4 / R);
     if (a.work_queue) {
         if (a.work_count <= 0) return MOE_OK;
         dim3 grid(ceil_div(units, 4), max(1, ceil_div(a.max_rows_hint, 64)), a.work_count);
         hipLaunchKernelGGL((expert_stream_queue_kernel<FMT, R, EPI>), grid, dim3(256), 0, stream, a);
+    } else if constexpr (EPI == EPI_SWIGLU_BF16 || EPI == EPI_ROWS_F32) {
+        if (a.waves_per_block == 0) {
+            dim3 grid(ceil_div(a.rows / 32, kWsConsumers), a.max_tiles);
+            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI>), grid, dim3(kWsThreads), 0, stream, a);
+        } else if (a.waves_per_block == 8) {
+            dim3 grid(ceil_div(units, 8), a.max_tiles);
+            hipLaunchKernelGGL((expert_stream_kernel<FMT, R, EPI, 8>), grid, dim3(512), 0, stream, a);
+        } else {
+            dim3 grid(ceil_div(units, 4), a.max_tiles);
+            hipLaunchKernelGGL((expert_stream_kernel<FMT, R, EPI, 4>), grid, dim3(256), 0, stream, a);
+        }
     } else {
-        dim3 grid(ceil_div(units, 4), a.max_tiles);
-        hipLaunchKernelGGL((expert_stream_kernel<FMT, R, EPI>), grid, dim3(256), 0, stream, a);
+        return MOE_ERR_FORMAT;
     }
     return launch_status();
 }
@@ -325,10 +635,10 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
 template <int FMT>
 int launch_fmt(const ExpertGemmArgs& a, int epi, hipStream_t stream) {
     switch (epi) {
-        case EPI_SWIGLU_BF16: return launch_cfg<FMT, 2, EPI_SWIGLU_BF16>(a, stream);
-        case EPI_ROWS_F32: return launch_cfg<FMT, 2, EPI_ROWS_F32>(a, stream);
-        case EPI_SWIGLU_F32: return launch_cfg<FMT, 2, EPI_SWIGLU_F32>(a, stream);
-        case EPI_SCATTER: return launch_cfg<FMT, 2, EPI_SCATTER>(a, stream);
+        case EPI_SWIGLU_BF16: return launch_cfg<FMT, EPI_SWIGLU_BF16>(a, stream);
+        case EPI_ROWS_F32: return launch_cfg<FMT, EPI_ROWS_F32>(a, stream);
+        case EPI_SWIGLU_F32: return launch_cfg<FMT, EPI_SWIGLU_F32>(a, stream);
+        case EPI_SCATTER: return launch_cfg<FMT, EPI_SCATTER>(a, stream);
     }
     return MOE_ERR_FORMAT;
 }
@@ -338,17 +648,11 @@ int launch_fmt(const ExpertGemmArgs& a, int epi, hipStream_t stream) {
 // epi: 0 fused gate/up (bf16 SwiGLU out), 1 fused down (fp32 rows per slot), 2 gate/up with fp32
 // in/out, 3 down with fp32 in and atomic scatter.  Token blocks hold at most 64 rows.
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream) {
-    if (a.rows % 64 != 0) return MOE_ERR_SHAPE;
+    if (a.rows % 64 != 0 || a.K % 32 != 0) return MOE_ERR_SHAPE;
     const bool queue = a.work_queue != nullptr;
     if (queue != (epi == EPI_SWIGLU_F32 || epi == EPI_SCATTER)) return MOE_ERR_FORMAT;
-    if (a.format == FMT_BF16) {
-        if (a.K % 64 != 0) return MOE_ERR_SHAPE;
-        return launch_fmt<FMT_BF16>(a, epi, stream);
-    }
-    if (a.format == FMT_MXFP4) {
-        if (a.K % 32 != 0) return MOE_ERR_SHAPE;
-        return launch_fmt<FMT_MXFP4>(a, epi, stream);
-    }
+    if (a.format == FMT_BF16) return launch_fmt<FMT_BF16>(a, epi, stream);
+    if (a.format == FMT_MXFP4) return launch_fmt<FMT_MXFP4>(a, epi, stream);
     return MOE_ERR_FORMAT;
 }
 

@@ -60,6 +60,7 @@ struct ExpertGemmArgs {
     float alpha, limit;
     int max_tiles;
     int format;
+    int waves_per_block;        // 0: warp-specialised kernel (6 consumer + 2 producer waves); 8 or 4: uniform waves
 };
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
 

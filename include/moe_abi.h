@@ -238,6 +238,20 @@ MOE_API size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int inter
                                  int experts_per_token);
 MOE_API int moe_block_forward(const moe_block_params* params, moe_stream_t stream);
 
+/* Per-stage timing of moe_block_forward with HIP events on the caller's stream.  Stands in for
+ * the reference's batch timing hooks, which its runtime calls but defines nowhere
+ * (reset_batch_timings / print_batch_timing_summary, src/getp/run.cpp:322, 326).
+ * Stages: 0 router partial dot products, 1 router finalise (top-k, softmax) + bf16 input copy,
+ * 2 bucketing, 3 gate/up GEMM + SwiGLU, 4 down GEMM, 5 combine.
+ * moe_block_forward_timed behaves like moe_block_forward and records MOE_N_STAGES + 1 events;
+ * moe_stage_timer_read waits for the last event and returns the stage durations in ms. */
+#define MOE_N_STAGES 6
+typedef struct moe_stage_timer moe_stage_timer;
+MOE_API int moe_stage_timer_create(moe_stage_timer** out);
+MOE_API void moe_stage_timer_destroy(moe_stage_timer* timer);
+MOE_API int moe_block_forward_timed(const moe_block_params* params, moe_stream_t stream, moe_stage_timer* timer);
+MOE_API int moe_stage_timer_read(moe_stage_timer* timer, float* stage_ms);
+
 /* ------------------------------------------------------------------------------------------
  * Synthetic workload generator (include/moe_synth.h), device side: fills device buffers with
  * the same values the host generator produces for (seed, tensor_id, index).
