@@ -14,8 +14,16 @@ constexpr size_t kAlign = 256;
 inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 inline hipStream_t as_stream(moe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
-// Token-block size of the expert kernels' tile map.
+// Token-block sizes of the expert kernels' tile map: decode-sized buckets / prefill-sized buckets.
 constexpr int kStreamTileTokens = 64;
+constexpr int kPrefillTileTokens = 128;
+
+// Prefill kernels once the average bucket fills most of a 128-token block.
+inline bool use_prefill_kernels(int T, int K, int E, unsigned flags) {
+    if (flags & MOE_FLAG_FORCE_STREAM) return false;
+    if (flags & MOE_FLAG_FORCE_TILED) return true;
+    return (long long)T * K >= 96LL * E;
+}
 
 // Carves the caller's workspace for moe_block_forward; with base == nullptr only sizes it.
 struct BlockWorkspace {
@@ -354,7 +362,10 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     if ((rc = mark())) return rc;
 
     // 2. bucketing + token-block map  (src/forward.cpp:329-376)
-    TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, kStreamTileTokens, ws.max_tiles};
+    const bool prefill = use_prefill_kernels(T, K, E, p->flags);
+    const int tile_tokens = prefill ? kPrefillTileTokens : kStreamTileTokens;
+    const int max_tiles = tile_map_capacity(T * K, E, tile_tokens);  // <= ws.max_tiles (sized for 64)
+    TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles};
     rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat, ws.slot_of,
                        map, stream);
     if (rc) return rc;
@@ -367,17 +378,17 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     g.tile_row0 = ws.tile_row0;
     g.tile_rows = ws.tile_rows;
     g.n_tiles = ws.n_tiles;
-    g.max_tiles = ws.max_tiles;
+    g.max_tiles = max_tiles;
     g.alpha = p->alpha;
     g.limit = p->swiglu_limit;
     g.format = fmt;
 
     // eight waves (256 weight rows) per block when that still yields enough blocks to fill the chip
-    const int est_tiles = std::max(ceil_div(T * K, kStreamTileTokens), std::min(E, T * K));
+    const int est_tiles = std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
     auto pick_waves = [&](int rows) { return ceil_div(rows / 32, 8) * est_tiles >= 512 ? 8 : 4; };
     // measured on MI355X at decode shapes: bf16 weights stream fastest with uniform waves, MXFP4
     // weights (four times the work per byte) with producer/consumer waves
-    auto pick_kernel = [&](int rows) { return fmt == MOE_WEIGHTS_BF16 ? pick_waves(rows) : 0; };
+    auto pick_kernel = [&](int rows) { return prefill ? 16 : (fmt == MOE_WEIGHTS_BF16 ? pick_waves(rows) : 0); };
 
     ExpertGemmArgs a1 = g;
     a1.w = p->w_mlp1;

@@ -116,13 +116,15 @@ MOE_DEVICE void stream_epilogue(const ExpertGemmArgs& a, const f32x4 (&acc)[R][N
 // (the reference's x_by_expert / gate_by_expert buffers) and are rounded to bf16 while staged.
 // `active` is false for the waves of a ragged last block that own no rows: they still stage
 // activations and take part in every barrier.
-template <int FMT, int R, int NT, int EPI, bool ACT_F32, int WAVES>
+template <int FMT, int R, int NT, int EPI, bool ACT_F32, int WAVES, int NTMAX = kNTMax>
 MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit,
                             bool active) {
     static_assert(WAVES == 4 || WAVES == 8, "a block has 4 or 8 waves");
     constexpr int kStagers = WAVES / 4;                       // waves that stage the same k-step
     constexpr int TS = (NT + kStagers - 1) / kStagers;        // token tiles staged per wave
     constexpr int kUnitsPerGroup = 4 / R;
+    constexpr int kStageBytes = kStageSteps * NTMAX * 1024;  // one LDS stage buffer
+    static_assert(NT <= NTMAX && TS * kStagers <= NTMAX, "token tiles must fit the LDS stage");
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int q = lane & 15;
@@ -175,7 +177,7 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
             b_src[i] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K + k_lane);
         }
     }
-    uint8_t* const lds_wr = lds + (size_t)(step_w * kNTMax + half_w) * 1024 + (size_t)lane * 16;
+    uint8_t* const lds_wr = lds + (size_t)(step_w * NTMAX + half_w) * 1024 + (size_t)lane * 16;
     const uint8_t* const lds_rd = lds + (size_t)lane * 16;
 
     // Everything inside the stage loops is branch-free (clamped addresses + selects instead of
@@ -200,10 +202,10 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
     auto stage_store = [&](int buf) {
 #pragma unroll
         for (int t = 0; t < TS; ++t)
-            *reinterpret_cast<u32x4*>(lds_wr + (size_t)buf * kLdsStageBytes + t * kStagers * 1024) = stg[t];
+            *reinterpret_cast<u32x4*>(lds_wr + (size_t)buf * kStageBytes + t * kStagers * 1024) = stg[t];
     };
     auto b_frag = [&](int buf, int j, int t) {
-        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)buf * kLdsStageBytes + (j * kNTMax + t) * 1024);
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)buf * kStageBytes + (j * NTMAX + t) * 1024);
     };
 
     if (!active) {
@@ -237,13 +239,12 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
             for (int r = 0; r < R; ++r) ar[slot][r] = *reinterpret_cast<const u32x4*>(a_ptr[r] + off);
         };
         auto step = [&](int buf, int j) {
-            u32x4 b[NT];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) b[t] = b_frag(buf, j, t);
+            for (int t = 0; t < NT; ++t) {
+                const u32x4 b = b_frag(buf, j, t);
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(ar[j][r], b[t], acc[r][t]);
+                for (int r = 0; r < R; ++r) acc[r][t] = mfma_16x16x32(ar[j][r], b, acc[r][t]);
+            }
         };
         stage_load(0);
         load_a(0, 0);
@@ -271,11 +272,11 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
             __syncthreads();
         }
     } else {
-        // A ring of four stages (one 128-bit load per row tile and stage), loads issued three stages
-        // ahead of their use; one scale word per row tile covers four stages and is fetched one
-        // quad ahead.  The stage count is padded to a multiple of four with all-zero stages (zero
+        // A ring of D stages (one 128-bit load per row tile and stage), loads issued D-1 stages ahead
+        // of their use; one scale word per row tile covers four stages and is fetched one quad
+        // ahead.  The stage count is padded to a multiple of four with all-zero stages (zero
         // weights against zero activations) to keep the loop uniform.
-        constexpr int D = 4;
+        constexpr int D = (R >= 4) ? 2 : 4;
         const int rem_groups = (K / 32) & 3;  // MX blocks in a ragged last stage (0 = none)
         const int n_quads = ceil_div(n_stages, 4);
         u32x4 araw[D][R];
@@ -295,25 +296,27 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
 #pragma unroll
             for (int r = 0; r < R; ++r) dst[r] = *reinterpret_cast<const uint32_t*>(s_ptr[r] + off);
         };
-        auto do_stage = [&](int slot, int s) {
+        auto do_stage = [&](int slot, int qpos, int s) {
             const int buf = s & 1;
             stage_load(s + 1);
             load_a((slot + D - 1) % D, s + D - 1);
             float sc[R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32((sw_cur[r] >> (8 * slot)) & 0xFFu);
+            for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32((sw_cur[r] >> (8 * qpos)) & 0xFFu);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                u32x4 b[NT];
-#pragma unroll
-                for (int t = 0; t < NT; ++t) b[t] = b_frag(buf, j, t);
+                u32x4 av[R];
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     uint32_t d[4];
                     mxfp4_dword_to_bf16x8(araw[slot][r][j], sc[r], d);
-                    const u32x4 av = {d[0], d[1], d[2], d[3]};
+                    av[r] = u32x4{d[0], d[1], d[2], d[3]};
+                }
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
+                for (int t = 0; t < NT; ++t) {
+                    const u32x4 b = b_frag(buf, j, t);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r][t] = mfma_16x16x32(av[r], b, acc[r][t]);
                 }
             }
             stage_store(buf ^ 1);
@@ -328,7 +331,7 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
         for (int qd = 0; qd < n_quads; ++qd) {
             load_scales(sw_nxt, qd + 1);
 #pragma unroll
-            for (int i = 0; i < D; ++i) do_stage(i, 4 * qd + i);
+            for (int i = 0; i < 4; ++i) do_stage(i % D, i, 4 * qd + i);
 #pragma unroll
             for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
         }
@@ -607,6 +610,167 @@ __global__ __launch_bounds__(256) void expert_stream_queue_kernel(ExpertGemmArgs
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Prefill-sized buckets: a 64-row x 128-token tile per wave (R = 4 row tiles, up to 8 token tiles),
+// so a weight operand — for MXFP4 dequantised once in registers — feeds eight MFMAs, and the LDS
+// holds the 128-token activation stage (2 x 32 KiB).  MXFP4 weights: activations are moved
+// global -> LDS by direct-to-LDS loads issued one stage ahead by all eight waves (no staging
+// registers), weights are fetched one stage ahead into registers.  bf16 weights reuse
+// stream_body with the same tile.
+// grid = (ceil(rows / 512), max_tiles), block = 512, token blocks of up to 128 rows.
+// ---------------------------------------------------------------------------------------------
+template <int NT, int EPI>
+MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit,
+                                   bool active) {
+    constexpr int R = 4;
+    constexpr int NTMAX = 8;
+    constexpr int kStageBytes = kStageSteps * NTMAX * 1024;
+    constexpr int TS = (NT + 1) / 2;  // token tiles staged per wave
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane & 15;
+    const int g = lane >> 4;
+    const int K = a.K;
+    const int G = K / 32;
+    const int n_stages = ceil_div(K, kStageElems);
+    const int n_quads = ceil_div(n_stages, 4);
+    const int rem_groups = G & 3;
+
+    // activation staging: this wave moves k-step wave%4 of token tiles wave/4, wave/4 + 2, ...
+    const int step_w = wave & 3;
+    const int half_w = wave >> 2;
+    const int k_lane = 32 * g + 8 * step_w;  // lane group g owns MX block g of a stage
+    const uint8_t* b_row[TS];
+#pragma unroll
+    for (int i = 0; i < TS; ++i) {
+        const int idx = min((half_w + 2 * i) * 16 + q, nrows - 1);
+        const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
+        b_row[i] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
+    }
+    auto issue_b = [&](int s) {
+        const int k = s * kStageElems + k_lane;
+        const size_t off = (k < K) ? (size_t)k * 2 : 0;  // past the row: re-read its start (weights are 0 there)
+        uint8_t* dst = lds + (size_t)(s & 1) * kStageBytes + (size_t)(step_w * NTMAX + half_w) * 1024;
+#pragma unroll
+        for (int i = 0; i < TS; ++i) dma16(b_row[i] + off, dst + i * 2048);
+    };
+    const uint8_t* const lds_rd = lds + (size_t)lane * 16;
+    auto b_frag = [&](int s, int j, int t) {
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & 1) * kStageBytes + (j * NTMAX + t) * 1024);
+    };
+
+    if (!active) {
+        issue_b(0);
+        wait_vmcnt<0>();
+        __syncthreads();
+        for (int s = 0; s < 4 * n_quads; ++s) {
+            issue_b(s + 1);
+            wait_vmcnt<0>();
+            __syncthreads();
+        }
+        return;
+    }
+
+    const size_t tile_bytes = (size_t)G * 256;
+    const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
+    const uint8_t* const a_base = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride +
+                                  (size_t)unit * 4 * tile_bytes + (size_t)lane * 16;
+    const uint8_t* const s_base = a.w_scales + (size_t)e * a.s_expert_stride + (size_t)unit * 4 * stile_bytes +
+                                  (size_t)lane * 4;
+    f32x4 acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    u32x4 araw[2][R];
+    uint32_t sw_cur[R], sw_nxt[R];
+    auto load_a = [&](int slot, int s) {
+        const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
+        const size_t off = live ? (size_t)s * 1024 : 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(a_base + r * tile_bytes + off);
+            araw[slot][r] = live ? v : u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+    auto load_scales = [&](uint32_t (&dst)[R], int quad) {
+        const size_t off = (size_t)min(quad, n_quads - 1) * 256;
+#pragma unroll
+        for (int r = 0; r < R; ++r) dst[r] = *reinterpret_cast<const uint32_t*>(s_base + r * stile_bytes + off);
+    };
+    auto do_stage = [&](int slot, int qpos, int s) {
+        issue_b(s + 1);
+        load_a(slot ^ 1, s + 1);
+        float sc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32((sw_cur[r] >> (8 * qpos)) & 0xFFu);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            u32x4 av[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                uint32_t d[4];
+                mxfp4_dword_to_bf16x8(araw[slot][r][j], sc[r], d);
+                av[r] = u32x4{d[0], d[1], d[2], d[3]};
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const u32x4 b = b_frag(s, j, t);
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r][t] = mfma_16x16x32(av[r], b, acc[r][t]);
+            }
+        }
+        wait_vmcnt<0>();  // next stage's activations (direct-to-LDS) and weights have landed
+        __syncthreads();
+    };
+    issue_b(0);
+    load_scales(sw_cur, 0);
+    load_a(0, 0);
+    wait_vmcnt<0>();
+    __syncthreads();
+    for (int qd = 0; qd < n_quads; ++qd) {
+        load_scales(sw_nxt, qd + 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) do_stage(i & 1, i, 4 * qd + i);
+#pragma unroll
+        for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
+    }
+    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, unit, 0);
+}
+
+template <int FMT, int NT, int EPI>
+MOE_DEVICE void prefill_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit, bool active) {
+    if constexpr (FMT == FMT_MXFP4) {
+        prefill_body_mxfp4<NT, EPI>(a, lds, e, row0, nrows, unit, active);
+    } else {
+        stream_body<FMT, 4, NT, EPI, false, 8, 8>(a, lds, e, row0, nrows, unit, active);
+    }
+}
+
+template <int FMT, int EPI>
+__global__ __launch_bounds__(512, 2) void expert_prefill_kernel(ExpertGemmArgs a) {
+    constexpr int NTMAX = 8;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageSteps * NTMAX * 1024];
+    const int tile = blockIdx.y;
+    if (tile >= *a.n_tiles) return;  // block-uniform
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int unit = blockIdx.x * 8 + wave;
+    const bool active = unit < a.rows / 64;
+    const int e = a.tile_expert[tile];
+    const int row0 = a.tile_row0[tile];
+    const int nrows = a.tile_rows[tile];
+    const int nt = (nrows + 15) >> 4;  // block-uniform
+    if (nt > 6) {
+        prefill_body<FMT, 8, EPI>(a, lds, e, row0, nrows, unit, active);
+    } else if (nt > 4) {
+        prefill_body<FMT, 6, EPI>(a, lds, e, row0, nrows, unit, active);
+    } else if (nt > 2) {
+        prefill_body<FMT, 4, EPI>(a, lds, e, row0, nrows, unit, active);
+    } else {
+        prefill_body<FMT, 2, EPI>(a, lds, e, row0, nrows, unit, active);
+    }
+}
+
 template <int FMT, int EPI>
 int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
     constexpr int R = 2;
@@ -616,7 +780,10 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
         dim3 grid(ceil_div(units, 4), max(1, ceil_div(a.max_rows_hint, 64)), a.work_count);
         hipLaunchKernelGGL((expert_stream_queue_kernel<FMT, R, EPI>), grid, dim3(256), 0, stream, a);
     } else if constexpr (EPI == EPI_SWIGLU_BF16 || EPI == EPI_ROWS_F32) {
-        if (a.waves_per_block == 0) {
+        if (a.waves_per_block == 16) {
+            dim3 grid(ceil_div(a.rows / 64, 8), a.max_tiles);
+            hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI>), grid, dim3(512), 0, stream, a);
+        } else if (a.waves_per_block == 0) {
             dim3 grid(ceil_div(a.rows / 32, kWsConsumers), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI>), grid, dim3(kWsThreads), 0, stream, a);
         } else if (a.waves_per_block == 8) {

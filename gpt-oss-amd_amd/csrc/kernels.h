@@ -60,7 +60,8 @@ struct ExpertGemmArgs {
     float alpha, limit;
     int max_tiles;
     int format;
-    int waves_per_block;        // 0: warp-specialised kernel (6 consumer + 2 producer waves); 8 or 4: uniform waves
+    int waves_per_block;        // kernel choice: 0 warp-specialised (10 consumer + 2 producer waves); 8 or 4 uniform
+                                // waves, 64-token blocks; 16 prefill kernel (8 waves, 128-token blocks)
 };
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
 
