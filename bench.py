@@ -31,10 +31,13 @@ def parse():
     ap.add_argument("--cpu-tokens", type=int, default=256, help="tokens of the workload the CPU baseline runs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--flags", type=int, default=0)
+    ap.add_argument("--graph", action="store_true",
+                    help="replay a captured HIP graph of one moe_block_forward call per step instead of plain launches "
+                         "(measured: no faster, the kernels' own dependent latencies dominate)")
     return ap.parse_args()
 
 
-def measure(pkg, wl, torch, shape, table, steps, warmup, flags=0):
+def measure(pkg, wl, torch, shape, table, steps, warmup, flags=0, use_graph=False):
     """Returns a dict of measurements for one workload on cuda:0."""
     dev = torch.device("cuda:0")
     blk, raw = wl.make_device_layer(shape, table, dev)
@@ -46,12 +49,30 @@ def measure(pkg, wl, torch, shape, table, steps, warmup, flags=0):
     p = blk.params(x, e_agg, topk_i, topk_v, flags=flags)
     stream = torch.cuda.current_stream().cuda_stream
 
-    for _ in range(warmup):
+    # One step = one moe_block_forward call.  The entry allocates nothing and never synchronises, so a
+    # serving loop can also capture it once and replay it (--graph).
+    for _ in range(3):
         blk.launch(p, stream)
+    torch.cuda.synchronize()
+    graph = None
+    if use_graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            blk.launch(p, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+
+    def step():
+        if graph is not None:
+            graph.replay()
+        else:
+            blk.launch(p, stream)
+
+    for _ in range(warmup):
+        step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        blk.launch(p, stream)
+        step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / steps
@@ -124,7 +145,7 @@ def main():
     table = oracle.normal_table()
 
     shape = wl.WORKLOADS[args.workload]
-    head = measure(pkg, wl, torch, shape, table, args.steps, args.warmup, args.flags)
+    head = measure(pkg, wl, torch, shape, table, args.steps, args.warmup, args.flags, args.graph)
     bound = "hbm" if shape.T <= 1024 else "mfma"
     if bound == "hbm":
         achieved = head["mlp1"]["bytes"] / (head["mlp1"]["ms"] * 1e-3) / 1e9
@@ -139,7 +160,7 @@ def main():
     also = []
     for name in [n for n in args.also.split(",") if n and n != args.workload]:
         r = measure(pkg, wl, torch, wl.WORKLOADS[name], table, max(10, args.steps // 4), max(3, args.warmup // 4),
-                    args.flags)
+                    args.flags, args.graph)
         also.append({k: r[k] for k in ("workload", "ms_per_step", "tokens_per_s", "block_hbm_frac", "block_mfma_frac",
                                        "stage_ms", "rows_per_expert_min_max")})
 
@@ -168,6 +189,7 @@ def main():
         "block_hbm_frac": head["block_hbm_frac"],
         "block_mfma_frac": head["block_mfma_frac"],
         "stage_ms": head["stage_ms"],
+        "launch": "HIP graph replay of one moe_block_forward call" if args.graph else "plain launches",
         "also": also,
     }
     print(json.dumps(out))

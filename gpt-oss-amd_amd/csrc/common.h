@@ -100,7 +100,9 @@ MOE_DEVICE float swiglu(float gate, float up, float alpha, float limit) {
     gate = gate > limit ? limit : gate;
     up = up > limit ? limit : up;
     up = up < -limit ? -limit : up;
-    const float sig = 1.0f / (1.0f + expf(-alpha * gate));
+    // exp through the hardware exp2 (relative error ~1e-6, far inside the 1e-2 output tolerance;
+    // the reference's own GPU kernel uses __expf as well, src/hip/moe.hip:189)
+    const float sig = 1.0f / (1.0f + __expf(-alpha * gate));
     return (gate * sig) * (up + 1.0f);
 }
 

@@ -619,13 +619,14 @@ __global__ __launch_bounds__(256) void expert_stream_queue_kernel(ExpertGemmArgs
 // stream_body with the same tile.
 // grid = (ceil(rows / 512), max_tiles), block = 512, token blocks of up to 128 rows.
 // ---------------------------------------------------------------------------------------------
-template <int NT, int EPI>
+template <int NT, int EPI, int WAVES>
 MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit,
                                    bool active) {
     constexpr int R = 4;
     constexpr int NTMAX = 8;
     constexpr int kStageBytes = kStageSteps * NTMAX * 1024;
-    constexpr int TS = (NT + 1) / 2;  // token tiles staged per wave
+    constexpr int kStagers = WAVES / 4;                 // waves that stage the same k-step
+    constexpr int TS = (NT + kStagers - 1) / kStagers;  // token tiles staged per wave
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int q = lane & 15;
@@ -636,14 +637,14 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     const int n_quads = ceil_div(n_stages, 4);
     const int rem_groups = G & 3;
 
-    // activation staging: this wave moves k-step wave%4 of token tiles wave/4, wave/4 + 2, ...
+    // activation staging: this wave moves k-step wave%4 of token tiles wave/4, wave/4 + WAVES/4, ...
     const int step_w = wave & 3;
     const int half_w = wave >> 2;
     const int k_lane = 32 * g + 8 * step_w;  // lane group g owns MX block g of a stage
     const uint8_t* b_row[TS];
 #pragma unroll
     for (int i = 0; i < TS; ++i) {
-        const int idx = min((half_w + 2 * i) * 16 + q, nrows - 1);
+        const int idx = min((half_w + kStagers * i) * 16 + q, nrows - 1);
         const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
         b_row[i] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
     }
@@ -652,7 +653,7 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
         const size_t off = (k < K) ? (size_t)k * 2 : 0;  // past the row: re-read its start (weights are 0 there)
         uint8_t* dst = lds + (size_t)(s & 1) * kStageBytes + (size_t)(step_w * NTMAX + half_w) * 1024;
 #pragma unroll
-        for (int i = 0; i < TS; ++i) dma16(b_row[i] + off, dst + i * 2048);
+        for (int i = 0; i < TS; ++i) dma16(b_row[i] + off, dst + i * kStagers * 1024);
     };
     const uint8_t* const lds_rd = lds + (size_t)lane * 16;
     auto b_frag = [&](int s, int j, int t) {
@@ -713,9 +714,15 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
                 mxfp4_dword_to_bf16x8(araw[slot][r][j], sc[r], d);
                 av[r] = u32x4{d[0], d[1], d[2], d[3]};
             }
+            // activation operands are read from LDS two token tiles ahead of the MFMAs that use them
+            u32x4 bq[2];
+            bq[0] = b_frag(s, j, 0);
+            if constexpr (NT > 1) bq[1] = b_frag(s, j, 1);
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                const u32x4 b = b_frag(s, j, t);
+                const u32x4 b = bq[t & 1];
+                if (t + 2 < NT) bq[t & 1] = b_frag(s, j, t + 2);
+                __builtin_amdgcn_sched_barrier(0);  // keep the read above ahead of the MFMAs below
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc[r][t] = mfma_16x16x32(av[r], b, acc[r][t]);
             }
@@ -738,36 +745,38 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, unit, 0);
 }
 
-template <int FMT, int NT, int EPI>
+template <int FMT, int NT, int EPI, int WAVES>
 MOE_DEVICE void prefill_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit, bool active) {
     if constexpr (FMT == FMT_MXFP4) {
-        prefill_body_mxfp4<NT, EPI>(a, lds, e, row0, nrows, unit, active);
+        prefill_body_mxfp4<NT, EPI, WAVES>(a, lds, e, row0, nrows, unit, active);
     } else {
-        stream_body<FMT, 4, NT, EPI, false, 8, 8>(a, lds, e, row0, nrows, unit, active);
+        stream_body<FMT, 4, NT, EPI, false, WAVES, 8>(a, lds, e, row0, nrows, unit, active);
     }
 }
 
-template <int FMT, int EPI>
-__global__ __launch_bounds__(512, 2) void expert_prefill_kernel(ExpertGemmArgs a) {
+// WAVES = 4: two blocks of four waves per CU (their barriers are independent, so one block's
+// stage hand-over overlaps the other's MFMAs); WAVES = 8: one block of eight.
+template <int FMT, int EPI, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 2) void expert_prefill_kernel(ExpertGemmArgs a) {
     constexpr int NTMAX = 8;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageSteps * NTMAX * 1024];
     const int tile = blockIdx.y;
     if (tile >= *a.n_tiles) return;  // block-uniform
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * 8 + wave;
+    const int unit = blockIdx.x * WAVES + wave;
     const bool active = unit < a.rows / 64;
     const int e = a.tile_expert[tile];
     const int row0 = a.tile_row0[tile];
     const int nrows = a.tile_rows[tile];
     const int nt = (nrows + 15) >> 4;  // block-uniform
     if (nt > 6) {
-        prefill_body<FMT, 8, EPI>(a, lds, e, row0, nrows, unit, active);
+        prefill_body<FMT, 8, EPI, WAVES>(a, lds, e, row0, nrows, unit, active);
     } else if (nt > 4) {
-        prefill_body<FMT, 6, EPI>(a, lds, e, row0, nrows, unit, active);
+        prefill_body<FMT, 6, EPI, WAVES>(a, lds, e, row0, nrows, unit, active);
     } else if (nt > 2) {
-        prefill_body<FMT, 4, EPI>(a, lds, e, row0, nrows, unit, active);
+        prefill_body<FMT, 4, EPI, WAVES>(a, lds, e, row0, nrows, unit, active);
     } else {
-        prefill_body<FMT, 2, EPI>(a, lds, e, row0, nrows, unit, active);
+        prefill_body<FMT, 2, EPI, WAVES>(a, lds, e, row0, nrows, unit, active);
     }
 }
 
@@ -781,8 +790,11 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
         hipLaunchKernelGGL((expert_stream_queue_kernel<FMT, R, EPI>), grid, dim3(256), 0, stream, a);
     } else if constexpr (EPI == EPI_SWIGLU_BF16 || EPI == EPI_ROWS_F32) {
         if (a.waves_per_block == 16) {
+            dim3 grid(ceil_div(a.rows / 64, 4), a.max_tiles);
+            hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 0, stream, a);
+        } else if (a.waves_per_block == 17) {
             dim3 grid(ceil_div(a.rows / 64, 8), a.max_tiles);
-            hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI>), grid, dim3(512), 0, stream, a);
+            hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 8>), grid, dim3(512), 0, stream, a);
         } else if (a.waves_per_block == 0) {
             dim3 grid(ceil_div(a.rows / 32, kWsConsumers), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI>), grid, dim3(kWsThreads), 0, stream, a);

@@ -12,7 +12,8 @@ namespace moe {
 // accumulator walks its segment in ascending k exactly like the reference loop; with one segment
 // the fp64 sum is bit-identical to src/run.cpp:348-351.  The four waves of a block share a
 // transposed activation chunk in LDS (row stride 65 floats: conflict-free for the transposing
-// store and for the lane-per-token read); weights are wave-uniform 16-byte loads.
+// store and for the lane-per-token read); weights are wave-uniform 16-byte loads issued one group
+// of eight elements ahead (scalar registers: no vector ALU work to unpack them).
 // grid = (ceil(T/64), ceil(E/(4*EG)), S), block = 256.
 // partial layout: [S][T][E] fp64.
 // ---------------------------------------------------------------------------------------------
@@ -26,7 +27,7 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const float* __rest
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t0 = blockIdx.x * 64;
-    const int e0 = (blockIdx.y * 4 + wave) * EG;
+    const int e0 = (blockIdx.y * 4 + wave) * EG;  // first expert of the wave
     const int s = blockIdx.z;
     const int kbeg = s * seg_len;
     const int kend = min(H, kbeg + seg_len);
@@ -35,28 +36,56 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const float* __rest
 #pragma unroll
     for (int j = 0; j < EG; ++j) acc[j] = 0.0;
 
-    for (int k0 = kbeg; k0 < kend; k0 += KC) {
+    // chunk c+1 is fetched into registers while chunk c is consumed from LDS
+    float4 xr[4];
+    auto fetch = [&](int k0) {
         const int kc = min(KC, kend - k0);  // multiple of 8
         const int q4 = kc >> 2;
-        for (int i = threadIdx.x; i < 64 * q4; i += 256) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int i = threadIdx.x + 256 * it;
             const int tl = i / q4;
             const int c = i - tl * q4;
             const int tok = t0 + tl;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (tok < T) v = *reinterpret_cast<const float4*>(x + (size_t)tok * H + k0 + 4 * c);
-            xs[4 * c + 0][tl] = v.x;
-            xs[4 * c + 1][tl] = v.y;
-            xs[4 * c + 2][tl] = v.z;
-            xs[4 * c + 3][tl] = v.w;
+            xr[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (i < 64 * q4 && tok < T) xr[it] = *reinterpret_cast<const float4*>(x + (size_t)tok * H + k0 + 4 * c);
         }
+    };
+    auto stash = [&](int k0) {
+        const int kc = min(KC, kend - k0);
+        const int q4 = kc >> 2;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int i = threadIdx.x + 256 * it;
+            if (i < 64 * q4) {
+                const int tl = i / q4;
+                const int c = i - tl * q4;
+                xs[4 * c + 0][tl] = xr[it].x;
+                xs[4 * c + 1][tl] = xr[it].y;
+                xs[4 * c + 2][tl] = xr[it].z;
+                xs[4 * c + 3][tl] = xr[it].w;
+            }
+        }
+    };
+    // weights: wave-uniform addresses (scalar loads), fetched one group of eight ahead
+    const uint16_t* wrow[EG];
+#pragma unroll
+    for (int j = 0; j < EG; ++j) wrow[j] = w + (size_t)min(e0 + j, E - 1) * H;
+    uint4 wv[EG], wn[EG];
+#pragma unroll
+    for (int j = 0; j < EG; ++j) wn[j] = *reinterpret_cast<const uint4*>(wrow[j] + min(kbeg, H - 8));
+    if (kbeg < kend) fetch(kbeg);
+    for (int k0 = kbeg; k0 < kend; k0 += KC) {
+        const int kc = min(KC, kend - k0);
+        stash(k0);
         __syncthreads();
+        if (k0 + KC < kend) fetch(k0 + KC);
         if (e0 < E) {
             for (int kk = 0; kk < kc; kk += 8) {
-                uint4 wv[EG];
 #pragma unroll
                 for (int j = 0; j < EG; ++j) {
-                    const int e = min(e0 + j, E - 1);
-                    wv[j] = *reinterpret_cast<const uint4*>(w + (size_t)e * H + k0 + kk);
+                    wv[j] = wn[j];
+                    wn[j] = *reinterpret_cast<const uint4*>(wrow[j] + min(k0 + kk + 8, H - 8));
                 }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
