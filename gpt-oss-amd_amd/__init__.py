@@ -284,7 +284,7 @@ class MoeBlock:
     router -> top-k -> softmax -> bucketing -> experts -> combine (src/forward.cpp:317-514)."""
 
     def __init__(self, H, I, E, K, w_router, b_router, w_mlp1, b_mlp1, w_mlp2, b_mlp2, max_tokens,
-                 w_mlp1_scales=None, w_mlp2_scales=None, swiglu_limit=7.0, alpha=1.702):
+                 w_mlp1_scales=None, w_mlp2_scales=None, swiglu_limit=7.0, alpha=1.702, workspace=None):
         self.H, self.I, self.E, self.K = H, I, E, K
         self.fmt = MOE_WEIGHTS_BF16 if w_mlp1_scales is None else MOE_WEIGHTS_MXFP4_TILED
         self.tensors = dict(w_router=w_router, b_router=b_router, w_mlp1=w_mlp1, b_mlp1=b_mlp1, w_mlp2=w_mlp2,
@@ -294,7 +294,11 @@ class MoeBlock:
         nbytes = block_workspace_bytes(max_tokens, H, I, E, K)
         if nbytes == 0:
             raise MoeError("moe_block_workspace_bytes", -2)
-        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=w_router.device)
+        if workspace is None:
+            workspace = torch.empty(nbytes, dtype=torch.uint8, device=w_router.device)
+        elif workspace.numel() < nbytes:
+            raise MoeError("moe_block_workspace_bytes", -4)
+        self.workspace = workspace  # layers run one after another on a stream may share it
 
     def params(self, t, e_agg, topk_i, topk_v, router_score=None, residual_x=None, flags=0):
         T = t.shape[0]

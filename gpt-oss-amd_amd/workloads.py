@@ -135,7 +135,7 @@ def fill_device(dims, kind, args, seed, table_d, device):
     return t
 
 
-def make_device_layer(shape, table_host, device, layer=0, keep_canonical=False):
+def make_device_layer(shape, table_host, device, layer=0, keep_canonical=False, workspace=None):
     """Weights of one layer in device memory, MXFP4 tensors repacked to the tiled layout.
     Returns (MoeBlock, dict of raw tensors)."""
     table_d = normal_table_device(table_host, device)
@@ -143,13 +143,13 @@ def make_device_layer(shape, table_host, device, layer=0, keep_canonical=False):
     if shape.fmt == "bf16":
         blk = _pkg.MoeBlock(shape.H, shape.I, shape.E, shape.K, raw["w_router"], raw["b_router"], raw["w_mlp1"],
                             raw["b_mlp1"], raw["w_mlp2"], raw["b_mlp2"], max_tokens=shape.T,
-                            swiglu_limit=shape.swiglu_limit, alpha=shape.alpha)
+                            swiglu_limit=shape.swiglu_limit, alpha=shape.alpha, workspace=workspace)
     else:
         t1b, t1s = _pkg.mxfp4_repack(raw["w_mlp1_blocks"], raw["w_mlp1_scales"])
         t2b, t2s = _pkg.mxfp4_repack(raw["w_mlp2_blocks"], raw["w_mlp2_scales"])
         blk = _pkg.MoeBlock(shape.H, shape.I, shape.E, shape.K, raw["w_router"], raw["b_router"], t1b, raw["b_mlp1"],
                             t2b, raw["b_mlp2"], max_tokens=shape.T, w_mlp1_scales=t1s, w_mlp2_scales=t2s,
-                            swiglu_limit=shape.swiglu_limit, alpha=shape.alpha)
+                            swiglu_limit=shape.swiglu_limit, alpha=shape.alpha, workspace=workspace)
         if not keep_canonical:
             torch.cuda.synchronize(device)
             for n in ("w_mlp1_blocks", "w_mlp1_scales", "w_mlp2_blocks", "w_mlp2_scales"):
@@ -160,6 +160,42 @@ def make_device_layer(shape, table_host, device, layer=0, keep_canonical=False):
 def make_device_input(shape, table_host, device):
     d, k, a = input_spec(shape)
     return fill_device(d, k, a, shape.seed, normal_table_device(table_host, device), device)
+
+
+class DeviceStack:
+    """shape.layers MoE layers resident in device memory with the reference's layer glue around each
+    block: t = rmsnorm(x) with unit weight (src/forward.cpp:315), x += moe(t) (src/forward.cpp:514)."""
+
+    def __init__(self, shape, table_host, device):
+        self.shape = shape
+        nbytes = _pkg.block_workspace_bytes(shape.T, shape.H, shape.I, shape.E, shape.K)
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self.blocks = []
+        for layer in range(shape.layers):
+            blk, raw = make_device_layer(shape, table_host, device, layer=layer, workspace=self.workspace)
+            del raw
+            self.blocks.append(blk)
+        self.rms_w = torch.ones(shape.H, dtype=torch.bfloat16, device=device)
+        T = shape.T
+        self.t = torch.empty((T, shape.H), dtype=torch.float32, device=device)
+        self.e_agg = torch.empty((T, shape.H), dtype=torch.float32, device=device)
+        self.topk_i = torch.empty((shape.layers, T, shape.K), dtype=torch.int32, device=device)
+        self.topk_v = torch.empty((shape.layers, T, shape.K), dtype=torch.float32, device=device)
+
+    def prepare(self, x):
+        """Parameter blocks for forward(x): built once so the timed loop does no Python tensor work."""
+        self.params = [blk.params(self.t, self.e_agg, self.topk_i[l], self.topk_v[l], residual_x=x)
+                       for l, blk in enumerate(self.blocks)]
+        self.x = x
+
+    def forward(self, stream=None, start=0, stop=None):
+        """x <- x + moe_l(rmsnorm(x)) for l = start .. stop-1 (all layers by default), in place on self.x."""
+        s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+        T, H = self.shape.T, self.shape.H
+        stop = len(self.blocks) if stop is None else stop
+        for l in range(start, stop):
+            _pkg.rmsnorm(self.t, self.x, self.rms_w, T, H, stream=s)
+            self.blocks[l].launch(self.params[l], s)
 
 
 # ---- algorithmic work per block (what roofline fractions are computed from) ----------------------

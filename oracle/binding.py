@@ -46,10 +46,10 @@ def _load():
         "oracle_f32_to_bf16": (None, [_vp, _ll, _vp]),
         "oracle_bucket": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
         "oracle_synth_normal_table": (None, [_vp]),
-        "oracle_synth_normal_f32": (None, [_vp, _ll, _vp, _f, _u, _u]),
-        "oracle_synth_normal_bf16": (None, [_vp, _ll, _vp, _f, _u, _u]),
-        "oracle_synth_bytes": (None, [_vp, _ll, _u, _u]),
-        "oracle_synth_range_bytes": (None, [_vp, _ll, _u, _u, _u, _u]),
+        "oracle_synth_normal_f32": (None, [_vp, _ll, _vp, _f, _u, _u, _ll]),
+        "oracle_synth_normal_bf16": (None, [_vp, _ll, _vp, _f, _u, _u, _ll]),
+        "oracle_synth_bytes": (None, [_vp, _ll, _u, _u, _ll]),
+        "oracle_synth_range_bytes": (None, [_vp, _ll, _u, _u, _u, _u, _ll]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -206,25 +206,26 @@ def normal_table():
     return _TABLE
 
 
-def synth_normal_f32(shape, scale, seed, tensor_id):
+def synth_normal_f32(shape, scale, seed, tensor_id, start=0):
+    """Elements start .. start+prod(shape)-1 of the stream (seed, tensor_id)."""
     out = np.empty(shape, dtype=np.float32)
-    _lib.oracle_synth_normal_f32(_p(out), out.size, _p(normal_table()), scale, seed, tensor_id)
+    _lib.oracle_synth_normal_f32(_p(out), out.size, _p(normal_table()), scale, seed, tensor_id, start)
     return out
 
 
-def synth_normal_bf16(shape, scale, seed, tensor_id):
+def synth_normal_bf16(shape, scale, seed, tensor_id, start=0):
     out = np.empty(shape, dtype=np.uint16)
-    _lib.oracle_synth_normal_bf16(_p(out), out.size, _p(normal_table()), scale, seed, tensor_id)
+    _lib.oracle_synth_normal_bf16(_p(out), out.size, _p(normal_table()), scale, seed, tensor_id, start)
     return out
 
 
-def synth_bytes(shape, seed, tensor_id):
+def synth_bytes(shape, seed, tensor_id, start=0):
     out = np.empty(shape, dtype=np.uint8)
-    _lib.oracle_synth_bytes(_p(out), out.size, seed, tensor_id)
+    _lib.oracle_synth_bytes(_p(out), out.size, seed, tensor_id, start)
     return out
 
 
-def synth_range_bytes(shape, seed, tensor_id, lo, span):
+def synth_range_bytes(shape, seed, tensor_id, lo, span, start=0):
     out = np.empty(shape, dtype=np.uint8)
-    _lib.oracle_synth_range_bytes(_p(out), out.size, seed, tensor_id, lo, span)
+    _lib.oracle_synth_range_bytes(_p(out), out.size, seed, tensor_id, lo, span, start)
     return out

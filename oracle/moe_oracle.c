@@ -359,28 +359,30 @@ ORACLE_API int oracle_bucket(const int* topk_i, const float* topk_v, int T, int 
 /* ---- synthetic inputs (include/moe_synth.h), host side -------------------------------- */
 ORACLE_API void oracle_synth_normal_table(float* table) { moe_synth_build_normal_table(table); }
 
+/* every generator fills dst[0..n) with the stream elements start .. start+n-1 */
 ORACLE_API void oracle_synth_normal_f32(float* dst, long long n, const float* table, float scale,
-                                        unsigned seed, unsigned tensor_id) {
+                                        unsigned seed, unsigned tensor_id, long long start) {
 #pragma omp parallel for
     for (long long i = 0; i < n; ++i)
-        dst[i] = moe_synth_normal_f32(table, scale, seed, tensor_id, (uint64_t)i);
+        dst[i] = moe_synth_normal_f32(table, scale, seed, tensor_id, (uint64_t)(start + i));
 }
 
 ORACLE_API void oracle_synth_normal_bf16(uint16_t* dst, long long n, const float* table, float scale,
-                                         unsigned seed, unsigned tensor_id) {
+                                         unsigned seed, unsigned tensor_id, long long start) {
 #pragma omp parallel for
     for (long long i = 0; i < n; ++i)
-        dst[i] = moe_synth_normal_bf16(table, scale, seed, tensor_id, (uint64_t)i);
+        dst[i] = moe_synth_normal_bf16(table, scale, seed, tensor_id, (uint64_t)(start + i));
 }
 
-ORACLE_API void oracle_synth_bytes(uint8_t* dst, long long n, unsigned seed, unsigned tensor_id) {
+ORACLE_API void oracle_synth_bytes(uint8_t* dst, long long n, unsigned seed, unsigned tensor_id,
+                                   long long start) {
 #pragma omp parallel for
-    for (long long i = 0; i < n; ++i) dst[i] = moe_synth_byte(seed, tensor_id, (uint64_t)i);
+    for (long long i = 0; i < n; ++i) dst[i] = moe_synth_byte(seed, tensor_id, (uint64_t)(start + i));
 }
 
 ORACLE_API void oracle_synth_range_bytes(uint8_t* dst, long long n, unsigned seed, unsigned tensor_id,
-                                         unsigned lo, unsigned span) {
+                                         unsigned lo, unsigned span, long long start) {
 #pragma omp parallel for
     for (long long i = 0; i < n; ++i)
-        dst[i] = moe_synth_range_byte(seed, tensor_id, (uint64_t)i, lo, span);
+        dst[i] = moe_synth_range_byte(seed, tensor_id, (uint64_t)(start + i), lo, span);
 }
