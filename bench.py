@@ -26,11 +26,14 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode256_bf16")
-    ap.add_argument("--also", default="decode256_mxfp4,prefill4096_mxfp4_zipf",
+    ap.add_argument("--also", default="decode256_mxfp4,prefill4096_mxfp4_zipf,stack120b_mxfp4",
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--cpu-tokens", type=int, default=256, help="tokens of the workload the CPU baseline runs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--flags", type=int, default=0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="first run five plain 1 GiB device-to-device copies (a kernel of known traffic: 1 GiB read, "
+                         "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
     ap.add_argument("--graph", action="store_true",
                     help="replay a captured HIP graph of one moe_block_forward call per step instead of plain launches "
                          "(measured: no faster, the kernels' own dependent latencies dominate)")
@@ -115,6 +118,34 @@ def measure(pkg, wl, torch, shape, table, steps, warmup, flags=0, use_graph=Fals
     return res
 
 
+def measure_stack(pkg, wl, torch, shape, table, steps, warmup):
+    """The 36-layer 120b-shaped stack: one step = all layers (rmsnorm -> MoE block -> residual)."""
+    dev = torch.device("cuda:0")
+    stack = wl.DeviceStack(shape, table, dev)
+    x = wl.make_device_input(shape, table, dev)
+    x0 = x.clone()
+    stack.prepare(x)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(warmup):
+        x.copy_(x0)
+        stack.forward(stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        stack.forward(stream)  # activations keep evolving; routing stays data-dependent and realistic
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    alg_bytes = wl.algorithmic_bytes(shape) * shape.layers
+    alg_flops = wl.algorithmic_flops(shape) * shape.layers
+    res = {"workload": shape.name, "ms_per_step": ms, "tokens_per_s": shape.T / (ms * 1e-3), "layers": shape.layers,
+           "block_hbm_frac": alg_bytes / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9),
+           "block_mfma_frac": alg_flops / (ms * 1e-3) / (MFMA_BF16_PEAK_TFLOPS * 1e12),
+           "weights_gb": round(shape.layers * shape.E * wl.weight_bytes_per_expert(shape) / 1e9, 2)}
+    del stack
+    torch.cuda.empty_cache()
+    return res
+
+
 def cpu_baseline(ge, wl, shape, n_tokens):
     """The CPU oracle on the first n_tokens of the workload, all host threads."""
     sys.path.insert(0, os.path.join(ge.ROOT, "tests"))
@@ -144,6 +175,15 @@ def main():
     oracle = ge.import_oracle()  # normal-quantile table of the synthetic generator + CPU baseline
     table = oracle.normal_table()
 
+    if args.copy_calibration:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
     shape = wl.WORKLOADS[args.workload]
     head = measure(pkg, wl, torch, shape, table, args.steps, args.warmup, args.flags, args.graph)
     bound = "hbm" if shape.T <= 1024 else "mfma"
@@ -159,6 +199,9 @@ def main():
 
     also = []
     for name in [n for n in args.also.split(",") if n and n != args.workload]:
+        if wl.WORKLOADS[name].layers > 1:
+            also.append(measure_stack(pkg, wl, torch, wl.WORKLOADS[name], table, max(3, args.steps // 20), 2))
+            continue
         r = measure(pkg, wl, torch, wl.WORKLOADS[name], table, max(10, args.steps // 4), max(3, args.warmup // 4),
                     args.flags, args.graph)
         also.append({k: r[k] for k in ("workload", "ms_per_step", "tokens_per_s", "block_hbm_frac", "block_mfma_frac",

@@ -617,7 +617,7 @@ __global__ __launch_bounds__(256) void expert_stream_queue_kernel(ExpertGemmArgs
 // global -> LDS by direct-to-LDS loads issued one stage ahead by all eight waves (no staging
 // registers), weights are fetched one stage ahead into registers.  bf16 weights reuse
 // stream_body with the same tile.
-// grid = (ceil(rows / 512), max_tiles), block = 512, token blocks of up to 128 rows.
+// grid = (ceil(rows / (64 WAVES)), max_tiles), token blocks of up to 128 rows.
 // ---------------------------------------------------------------------------------------------
 template <int NT, int EPI, int WAVES>
 MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit,
@@ -760,10 +760,13 @@ template <int FMT, int EPI, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, 2) void expert_prefill_kernel(ExpertGemmArgs a) {
     constexpr int NTMAX = 8;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageSteps * NTMAX * 1024];
+    // Row block fastest: neighbouring blocks share one token block's activations, which measured
+    // faster than the order that keeps an expert's token blocks (same weights) together on one XCD.
     const int tile = blockIdx.y;
+    const int row_block = blockIdx.x;
     if (tile >= *a.n_tiles) return;  // block-uniform
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * WAVES + wave;
+    const int unit = row_block * WAVES + wave;
     const bool active = unit < a.rows / 64;
     const int e = a.tile_expert[tile];
     const int row0 = a.tile_row0[tile];
