@@ -146,6 +146,28 @@ def measure_stack(pkg, wl, torch, shape, table, steps, warmup):
     return res
 
 
+def profiled_traffic(root, workload, kernel_prefix):
+    """HBM-side bytes per launch of the dominant kernel from the committed rocprofv3 counter summary
+    (profiles/moe_block_<workload>.txt): 2 x FETCH_SIZE + WRITE_SIZE in KiB, the factors coming from
+    the plain-copy calibration recorded in that file.  None when no summary covers the workload."""
+    path = os.path.join(root, "profiles", "moe_block_%s.txt" % workload)
+    if not os.path.exists(path):
+        return None
+    section, vals = None, {}
+    for line in open(path):
+        if line.startswith("== FETCH_SIZE"):
+            section = "fetch"
+        elif line.startswith("== WRITE_SIZE"):
+            section = "write"
+        elif line.startswith("=="):
+            section = None
+        elif section and line.startswith(kernel_prefix) and section not in vals:
+            vals[section] = float(line.split("avg")[-1])
+    if "fetch" not in vals or "write" not in vals:
+        return None
+    return (2.0 * vals["fetch"] + vals["write"]) * 1024.0
+
+
 def cpu_baseline(ge, wl, shape, n_tokens):
     """The CPU oracle on the first n_tokens of the workload, all host threads."""
     sys.path.insert(0, os.path.join(ge.ROOT, "tests"))
@@ -187,15 +209,24 @@ def main():
     shape = wl.WORKLOADS[args.workload]
     head = measure(pkg, wl, torch, shape, table, args.steps, args.warmup, args.flags, args.graph)
     bound = "hbm" if shape.T <= 1024 else "mfma"
+    # the gate/up GEMM launch: which kernel serves it depends on bucket size and weight format
+    if shape.T * shape.K >= 96 * shape.E:
+        kname = "expert_prefill_kernel<%d, 0" % (0 if shape.fmt == "bf16" else 1)
+    elif shape.fmt == "bf16":
+        kname = "expert_stream_kernel<0, 2, 0"
+    else:
+        kname = "expert_stream_ws_kernel<1, 0"
+    traffic = profiled_traffic(ge.ROOT, shape.name, kname)
     if bound == "hbm":
         achieved = head["mlp1"]["bytes"] / (head["mlp1"]["ms"] * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "expert_stream_kernel (gate/up GEMM + SwiGLU)", "achieved": achieved,
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None}
+        roofline = {"bound": "hbm", "kernel": kname + "...> (gate/up GEMM + SwiGLU)", "achieved": achieved,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                    "algorithmic_bytes": head["mlp1"]["bytes"], "kernel_ms": head["mlp1"]["ms"]}
     else:
         achieved = head["mlp1"]["flops"] / (head["mlp1"]["ms"] * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": "gate/up GEMM + SwiGLU", "achieved": achieved,
+        roofline = {"bound": "mfma", "kernel": kname + "...> (gate/up GEMM + SwiGLU)", "achieved": achieved,
                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                    "traffic": None}
+                    "traffic": traffic, "algorithmic_flops": head["mlp1"]["flops"], "kernel_ms": head["mlp1"]["ms"]}
 
     also = []
     for name in [n for n in args.also.split(",") if n and n != args.workload]:

@@ -112,3 +112,18 @@ def test_zipf_router_bias(wl):
     b = (bits.astype(np.uint32) << 16).view(np.float32)
     assert b.max() == 0.0 and len(np.unique(b)) == shape.E
     assert abs(b.min() - wl.ZIPF_BETA * -1.2 * np.log(32)) < 0.02
+
+
+def test_cpp_host_headers_compile_link_and_check_arguments(pkg, tmp_path):
+    """The C++ host side (drop-in wrappers under the reference's function names + the layer
+    function) builds with a plain C++17 compiler against the C ABI and rejects null buffers."""
+    import subprocess
+    host = os.path.join(ROOT, "gpt-oss-amd_amd", "host")
+    exe = str(tmp_path / "example_layer_loop")
+    libdir = os.path.dirname(pkg.LIB_PATH)
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-o", exe,
+                    os.path.join(host, "example_layer_loop.cpp"), "-L" + libdir, "-lmoe_gfx950",
+                    "-Wl,-rpath," + libdir], check=True, capture_output=True)
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "workspace for B=256" in r.stdout
