@@ -13,7 +13,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmoe_gfx950.so")
+# MOE_GFX950_LIB selects another build of the same library (A/B timing of two builds in one session)
+LIB_PATH = os.environ.get("MOE_GFX950_LIB") or os.path.join(_HERE, "libmoe_gfx950.so")
 
 MOE_WEIGHTS_BF16 = 0
 MOE_WEIGHTS_MXFP4_TILED = 1

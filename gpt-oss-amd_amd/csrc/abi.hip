@@ -112,7 +112,7 @@ int moe_gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, cons
     if (!scratch || ((uintptr_t)scratch & 7u) || scratch_bytes < (size_t)S * N * M * sizeof(double))
         return MOE_ERR_WORKSPACE;
     double* partial = static_cast<double*>(scratch);
-    int rc = launch_router_partial(x_batch, w, partial, N, K, M, S, as_stream(stream));
+    int rc = launch_router_partial(x_batch, w, partial, nullptr, N, K, M, S, as_stream(stream));
     if (rc) return rc;
     return launch_router_finalize(partial, S, nullptr, bias, xout, nullptr, nullptr, N, M, 0, 0, 0, as_stream(stream));
 }
@@ -351,13 +351,11 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
 
     // 1. router logits -> top-k -> softmax  (src/forward.cpp:318-327; src/run.cpp:630-642)
     const int S = router_segments(T, E, H, (p->flags & MOE_FLAG_ROUTER_STRICT_ORDER) != 0);
-    rc = launch_router_partial(p->t, p->w_router, ws.router_partial, T, H, E, S, stream);
+    rc = launch_router_partial(p->t, p->w_router, ws.router_partial, ws.t_bf16, T, H, E, S, stream);
     if (rc) return rc;
     if ((rc = mark())) return rc;
     rc = launch_router_finalize(ws.router_partial, S, nullptr, p->b_router, p->router_score, p->topk_v, p->topk_i, T, E,
                                 K, 1, 1, stream);
-    if (rc) return rc;
-    rc = launch_convert_f32_bf16(p->t, ws.t_bf16, (size_t)T * H, stream);
     if (rc) return rc;
     if ((rc = mark())) return rc;
 

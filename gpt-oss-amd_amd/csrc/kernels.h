@@ -8,13 +8,12 @@ namespace moe {
 
 // ---- router.hip -------------------------------------------------------------------------------
 int router_segments(int T, int E, int H, bool strict);
-int launch_router_partial(const float* x, const uint16_t* w, double* partial, int T, int H, int E, int S,
-                          hipStream_t stream);
+int launch_router_partial(const float* x, const uint16_t* w, double* partial, uint16_t* x_bf16, int T, int H,
+                          int E, int S, hipStream_t stream);
 int launch_router_finalize(const double* partial, int S, const float* scores_in, const uint16_t* bias,
                            float* scores_out, float* topk_v, int* topk_i, int T, int E, int K, int do_topk,
                            int do_softmax, hipStream_t stream);
 int launch_softmax_rows(float* x, int B, int size, hipStream_t stream);
-int launch_convert_f32_bf16(const float* in, uint16_t* out, size_t n, hipStream_t stream);
 
 // ---- bucket.hip -------------------------------------------------------------------------------
 // Token-block map consumed by the expert kernels: tile i covers rows
