@@ -368,33 +368,49 @@ MOE_DEVICE void dma16(const void* gsrc, uint8_t* lds_dst_wave_uniform) {
 template <int FMT>
 MOE_DEVICE int ws_padded_stages(int K) {
     const int n_stages = ceil_div(K, kStageElems);
-    return (FMT == FMT_BF16) ? ceil_div(n_stages, 2) * 2 : ceil_div(n_stages, 6) * 6;
+    return (FMT == FMT_BF16) ? ceil_div(n_stages, 2) * 2 : ceil_div(n_stages, 4) * 4;
+}
+
+// LDS image of one stage of activations: token tile t at t*4096, row q (0..15) of the tile at
+// q*256, and inside the row the sixteen 16-byte chunks of the stage's 128 contraction elements,
+// chunk c stored at position c ^ q.  A producer instruction moves four rows of 256 contiguous
+// bytes (whole cache lines, each fetched once); the XOR spreads the sixteen rows that one
+// fragment read touches over all LDS banks.
+template <int FMT>
+MOE_DEVICE int ws_chunk(int j, int g) {  // chunk holding the operand of MFMA step j for lane group g
+    return (FMT == FMT_BF16) ? 4 * j + g : 4 * g + j;
 }
 
 template <int FMT, int NT>
 MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int nrows, int p) {
     constexpr int Q = 2 * NT;  // direct-to-LDS loads per stage issued by this wave
     const int lane = threadIdx.x & 63;
-    const int q = lane & 15;
-    const int g = lane >> 4;
+    const int pos = lane & 15;   // chunk position inside the row's LDS image
+    const int sub = lane >> 4;   // row inside the instruction's block of four
     const int K = a.K;
     const int n_pad = ws_padded_stages<FMT>(K);
-    const uint8_t* row[NT];
+    // this wave moves row blocks 2p and 2p+1 (rows 8p .. 8p+7) of every token tile
+    const uint8_t* row[NT][2];
+    int chunk[2];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        const int idx = min(t * 16 + q, nrows - 1);
-        const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
-        row[t] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
+    for (int ii = 0; ii < 2; ++ii) {
+        const int q = 4 * (2 * p + ii) + sub;
+        chunk[ii] = pos ^ q;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int idx = min(t * 16 + q, nrows - 1);
+            const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
+            row[t][ii] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
+        }
     }
     auto issue = [&](int s) {
         uint8_t* slot = lds + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes;
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-            const int j = 2 * p + jj;
-            const int k = (FMT == FMT_BF16) ? (s * kStageElems + 32 * j + 8 * g) : (s * kStageElems + 32 * g + 8 * j);
+        for (int ii = 0; ii < 2; ++ii) {
+            const int k = s * kStageElems + 8 * chunk[ii];
             const size_t off = (k < K) ? (size_t)k * 2 : 0;  // a position past the row re-reads its start
 #pragma unroll
-            for (int t = 0; t < NT; ++t) dma16(row[t] + off, slot + (j * kNTMax + t) * 1024);
+            for (int t = 0; t < NT; ++t) dma16(row[t][ii] + off, slot + t * 4096 + (2 * p + ii) * 1024);
         }
     };
     issue(0);
@@ -426,10 +442,10 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     }
     const int group = unit >> 1;
     const int r0 = (unit & 1) * R;
-    const uint8_t* const lds_rd = lds + (size_t)lane * 16;
+    const uint8_t* const lds_rd = lds + (size_t)q * 256;
     auto b_frag = [&](int s, int j, int t) {
-        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes +
-                                               (j * kNTMax + t) * 1024);
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes + t * 4096 +
+                                               ((ws_chunk<FMT>(j, g) ^ q) << 4));
     };
     f32x4 acc[R][NT];
 #pragma unroll
@@ -479,44 +495,64 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
             }
         }
     } else {
-        constexpr int D = 6;  // ring of stages: one 128-bit load + one scale byte per row tile and stage
+        // Weights: a ring of four stages (one 128-bit load per row tile and stage, issued three
+        // stages ahead of its use); scales: one word per row tile covers four stages and is
+        // fetched one group of four ahead.  Addresses are a wave-uniform base (scalar registers)
+        // plus a per-lane 32-bit offset that never changes, so a stage costs scalar arithmetic
+        // only.  Nothing touches a loaded value before the stage that consumes it: an instruction
+        // on it at load time would pin the wait for the load to the stage that issued it.
+        constexpr int D = 4;
         const int G = K / 32;
         const int rem_groups = G & 3;  // MX blocks in a ragged last stage (0 = none)
+        const int n_quads = n_pad / 4;
         const size_t tile_bytes = (size_t)G * 256;
         const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
         const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
         const uint8_t* sbase = a.w_scales + (size_t)e * a.s_expert_stride;
-        const uint8_t* a_ptr[R];
-        const uint8_t* s_ptr[R];
+        const uint8_t* wtile[R];  // wave-uniform
+        const uint8_t* stile[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const size_t tile = (size_t)group * 4 + (r0 + r);
-            a_ptr[r] = wbase + tile * tile_bytes + (size_t)lane * 16;
-            s_ptr[r] = sbase + tile * stile_bytes + (size_t)lane * 4;
+            wtile[r] = wbase + tile * tile_bytes;
+            stile[r] = sbase + tile * stile_bytes;
         }
+        const uint32_t voff_w = (uint32_t)lane * 16;
+        // ragged last stage: a lane group past the last MX block re-reads block 0 and gets scale 0
+        const uint32_t voff_w_ragged = (uint32_t)((g < rem_groups ? lane : q) * 16);
+        const uint32_t voff_s = (uint32_t)lane * 4;
+        const int last_quad = ceil_div(n_stages, 4) - 1;
         u32x4 araw[D][R];
-        uint32_t sbyte[D][R];
+        uint32_t sw_cur[R], sw_nxt[R];
         auto load_a = [&](int slot, int s) {
-            const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
-            const int sc = live ? s : 0;  // a dead lane group re-reads a block that exists and drops it
+            const int su = s < n_stages ? s : 0;  // a padding stage re-reads stage 0 and gets scale 0
+            const bool ragged = rem_groups != 0 && su == n_stages - 1;
+            const uint32_t vo = ragged ? voff_w_ragged : voff_w;
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[r] + (size_t)sc * 1024);
-                araw[slot][r] = live ? v : u32x4{0u, 0u, 0u, 0u};
-                sbyte[slot][r] = *(s_ptr[r] + (size_t)(sc >> 2) * 256 + (sc & 3));
-            }
+            for (int r = 0; r < R; ++r)
+                araw[slot][r] = *reinterpret_cast<const u32x4*>(wtile[r] + (size_t)su * 1024 + vo);
         };
+        auto load_scales = [&](uint32_t (&dst)[R], int quad) {
+            const size_t off = (size_t)min(quad, last_quad) * 256;
+#pragma unroll
+            for (int r = 0; r < R; ++r) dst[r] = *reinterpret_cast<const uint32_t*>(stile[r] + off + voff_s);
+        };
+        load_scales(sw_cur, 0);
 #pragma unroll
         for (int i = 0; i < D - 1; ++i) load_a(i, i);
         __syncthreads();
-        for (int s0 = 0; s0 < n_pad; s0 += D) {
+        for (int qd = 0; qd < n_quads; ++qd) {
+            load_scales(sw_nxt, qd + 1);
 #pragma unroll
-            for (int u = 0; u < D; ++u) {
-                const int s = s0 + u;
-                load_a((u + D - 1) % D, s + D - 1);
+            for (int i = 0; i < 4; ++i) {
+                const int s = 4 * qd + i;
+                load_a((i + D - 1) % D, s + D - 1);
+                __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three stages ahead of their use
+                const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
                 float sc[R];
 #pragma unroll
-                for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32(sbyte[u][r]);
+                for (int r = 0; r < R; ++r)
+                    sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu) : 0.0f;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     u32x4 b[NT];
@@ -525,7 +561,7 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
                         uint32_t d[4];
-                        mxfp4_dword_to_bf16x8(araw[u][r][j], sc[r], d);
+                        mxfp4_dword_to_bf16x8(araw[i][r][j], sc[r], d);
                         const u32x4 av = {d[0], d[1], d[2], d[3]};
 #pragma unroll
                         for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
@@ -533,6 +569,8 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
                 }
                 __syncthreads();
             }
+#pragma unroll
+            for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
         }
     }
     stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0);
