@@ -386,7 +386,18 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     auto pick_waves = [&](int rows) { return ceil_div(rows / 32, 8) * est_tiles >= 512 ? 8 : 4; };
     // measured on MI355X at decode shapes: bf16 weights stream fastest with uniform waves, MXFP4
     // weights (four times the work per byte) with producer/consumer waves
-    auto pick_kernel = [&](int rows) { return prefill ? 16 : (fmt == MOE_WEIGHTS_BF16 ? pick_waves(rows) : 0); };
+    // MXFP4 (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of 32 rows each.
+    // Blocks run in rounds of one per CU, so the cheaper choice is the one with the smaller
+    // rounds x rows-per-block product; more rows per block also re-read the activations less.
+    auto pick_consumers = [&](int rows) {
+        const int kCUs = 256;  // MI355X
+        const int cost10 = ceil_div(ceil_div(rows / 32, 10) * est_tiles, kCUs) * 10;
+        const int cost12 = ceil_div(ceil_div(rows / 32, 12) * est_tiles, kCUs) * 12;
+        return cost12 <= cost10 ? 1 : 0;
+    };
+    auto pick_kernel = [&](int rows) {
+        return prefill ? 16 : (fmt == MOE_WEIGHTS_BF16 ? pick_waves(rows) : pick_consumers(rows));
+    };
 
     ExpertGemmArgs a1 = g;
     a1.w = p->w_mlp1;

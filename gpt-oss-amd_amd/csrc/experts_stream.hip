@@ -341,18 +341,15 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
 }
 
 // ---------------------------------------------------------------------------------------------
-// Warp-specialised variant used by the fused block: a block has ten consumer waves (R = 2 row
-// tiles each, 320 weight rows per block) and two producer waves.  Producers move the bucket's
+// Producer/consumer variant used by the fused block: a block has CONS consumer waves (R = 2 row
+// tiles each, 32 CONS weight rows per block) and two producer waves.  Producers move the bucket's
 // activation rows global -> LDS with direct-to-LDS 128-bit loads (no registers, a ring of four
 // 16 KiB stage slots, three stages ahead of the consumers); consumers only have weight loads in
-// their memory queue, eight units (bf16: k-steps, MXFP4: stages) ahead of their use.  One barrier
-// per stage; every wave of the block executes exactly 1 + n_pad barriers.
+// their memory queue.  One barrier per stage; every wave of the block executes exactly
+// 1 + n_pad barriers.
 // Positions of the contraction range that do not exist (ragged last stage, padding stages) carry
 // a weight operand of exact zeros; the activation operand there is a clamped re-read of real data.
 // ---------------------------------------------------------------------------------------------
-constexpr int kWsConsumers = 10;
-constexpr int kWsProducers = 2;
-constexpr int kWsThreads = (kWsConsumers + kWsProducers) * 64;
 constexpr int kWsRing = 4;
 
 template <int N>
@@ -381,20 +378,21 @@ MOE_DEVICE int ws_chunk(int j, int g) {  // chunk holding the operand of MFMA st
     return (FMT == FMT_BF16) ? 4 * j + g : 4 * g + j;
 }
 
-template <int FMT, int NT>
+template <int FMT, int NT, int PROD>
 MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int nrows, int p) {
-    constexpr int Q = 2 * NT;  // direct-to-LDS loads per stage issued by this wave
+    constexpr int BP = 4 / PROD;  // four-row blocks of a token tile moved by this wave
+    constexpr int Q = BP * NT;    // direct-to-LDS loads per stage issued by this wave
     const int lane = threadIdx.x & 63;
     const int pos = lane & 15;   // chunk position inside the row's LDS image
     const int sub = lane >> 4;   // row inside the instruction's block of four
     const int K = a.K;
     const int n_pad = ws_padded_stages<FMT>(K);
-    // this wave moves row blocks 2p and 2p+1 (rows 8p .. 8p+7) of every token tile
-    const uint8_t* row[NT][2];
-    int chunk[2];
+    // this wave moves row blocks BP*p .. BP*p + BP-1 of every token tile
+    const uint8_t* row[NT][BP];
+    int chunk[BP];
 #pragma unroll
-    for (int ii = 0; ii < 2; ++ii) {
-        const int q = 4 * (2 * p + ii) + sub;
+    for (int ii = 0; ii < BP; ++ii) {
+        const int q = 4 * (BP * p + ii) + sub;
         chunk[ii] = pos ^ q;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -406,11 +404,11 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
     auto issue = [&](int s) {
         uint8_t* slot = lds + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes;
 #pragma unroll
-        for (int ii = 0; ii < 2; ++ii) {
+        for (int ii = 0; ii < BP; ++ii) {
             const int k = s * kStageElems + 8 * chunk[ii];
             const size_t off = (k < K) ? (size_t)k * 2 : 0;  // a position past the row re-reads its start
 #pragma unroll
-            for (int t = 0; t < NT; ++t) dma16(row[t][ii] + off, slot + t * 4096 + (2 * p + ii) * 1024);
+            for (int t = 0; t < NT; ++t) dma16(row[t][ii] + off, slot + t * 4096 + (BP * p + ii) * 1024);
         }
     };
     issue(0);
@@ -576,10 +574,10 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0);
 }
 
-// grid = (ceil(row units / 10), max_tiles), block = 768 (waves 0-9 consume, 10-11 produce); three
-// waves per SIMD, i.e. one block per CU with up to 168 registers per lane.
-template <int FMT, int EPI>
-__global__ __launch_bounds__(kWsThreads, 3) void expert_stream_ws_kernel(ExpertGemmArgs a) {
+// grid = (ceil(row units / CONS), max_tiles), block = 64 (CONS + PROD); one block per CU: twelve
+// waves leave 168 registers per lane, fourteen leave 128.
+template <int FMT, int EPI, int CONS, int PROD>
+__global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) void expert_stream_ws_kernel(ExpertGemmArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kWsRing * kLdsStageBytes];
     const int tile = blockIdx.y;
     if (tile >= *a.n_tiles) return;  // block-uniform
@@ -588,14 +586,14 @@ __global__ __launch_bounds__(kWsThreads, 3) void expert_stream_ws_kernel(ExpertG
     const int row0 = a.tile_row0[tile];
     const int nrows = a.tile_rows[tile];
     const int nt = (nrows + 15) >> 4;  // block-uniform
-    if (wave >= kWsConsumers) {
-        const int p = wave - kWsConsumers;
-        if (nt == 4) ws_producer<FMT, 4>(a, lds, row0, nrows, p);
-        else if (nt == 3) ws_producer<FMT, 3>(a, lds, row0, nrows, p);
-        else if (nt == 2) ws_producer<FMT, 2>(a, lds, row0, nrows, p);
-        else ws_producer<FMT, 1>(a, lds, row0, nrows, p);
+    if (wave >= CONS) {
+        const int p = wave - CONS;
+        if (nt == 4) ws_producer<FMT, 4, PROD>(a, lds, row0, nrows, p);
+        else if (nt == 3) ws_producer<FMT, 3, PROD>(a, lds, row0, nrows, p);
+        else if (nt == 2) ws_producer<FMT, 2, PROD>(a, lds, row0, nrows, p);
+        else ws_producer<FMT, 1, PROD>(a, lds, row0, nrows, p);
     } else {
-        const int unit = blockIdx.x * kWsConsumers + wave;
+        const int unit = blockIdx.x * CONS + wave;
         const bool active = unit < a.rows / 32;
         if (nt == 4) ws_consumer<FMT, 4, EPI>(a, lds, e, row0, nrows, unit, active);
         else if (nt == 3) ws_consumer<FMT, 3, EPI>(a, lds, e, row0, nrows, unit, active);
@@ -837,8 +835,15 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             dim3 grid(ceil_div(a.rows / 64, 8), a.max_tiles);
             hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 8>), grid, dim3(512), 0, stream, a);
         } else if (a.waves_per_block == 0) {
-            dim3 grid(ceil_div(a.rows / 32, kWsConsumers), a.max_tiles);
-            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI>), grid, dim3(kWsThreads), 0, stream, a);
+            dim3 grid(ceil_div(a.rows / 32, 10), a.max_tiles);
+            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, a);
+        } else if (a.waves_per_block == 1) {
+            if constexpr (FMT == FMT_MXFP4) {
+                dim3 grid(ceil_div(a.rows / 32, 12), a.max_tiles);
+                hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, a);
+            } else {
+                return MOE_ERR_FORMAT;
+            }
         } else if (a.waves_per_block == 8) {
             dim3 grid(ceil_div(units, 8), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_kernel<FMT, R, EPI, 8>), grid, dim3(512), 0, stream, a);

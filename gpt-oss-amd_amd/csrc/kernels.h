@@ -59,8 +59,9 @@ struct ExpertGemmArgs {
     float alpha, limit;
     int max_tiles;
     int format;
-    int waves_per_block;        // kernel choice: 0 warp-specialised (10 consumer + 2 producer waves); 8 or 4 uniform
-                                // waves, 64-token blocks; 16 prefill kernel (8 waves, 128-token blocks)
+    int waves_per_block;        // kernel choice: 0 / 1 producer-consumer kernel with 10 / 12 consumer waves (+ 2
+                                // producers); 8 or 4 uniform waves, 64-token blocks; 16 / 17 prefill kernel
+                                // (4 / 8 waves, 128-token blocks)
 };
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
 
