@@ -396,7 +396,7 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
         return cost12 <= cost10 ? 1 : 0;
     };
     auto pick_kernel = [&](int rows) {
-        return prefill ? 16 : (fmt == MOE_WEIGHTS_BF16 ? pick_waves(rows) : pick_consumers(rows));
+        return prefill ? 16 : pick_consumers(rows);
     };
 
     ExpertGemmArgs a1 = g;

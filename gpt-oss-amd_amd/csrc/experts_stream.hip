@@ -375,7 +375,7 @@ MOE_DEVICE int ws_padded_stages(int K) {
 // fragment read touches over all LDS banks.
 template <int FMT>
 MOE_DEVICE int ws_chunk(int j, int g) {  // chunk holding the operand of MFMA step j for lane group g
-    return (FMT == FMT_BF16) ? 4 * j + g : 4 * g + j;
+    return (FMT == FMT_BF16) ? 8 * (j >> 1) + 2 * g + (j & 1) : 4 * g + j;
 }
 
 template <int FMT, int NT, int PROD>
@@ -452,42 +452,55 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     if constexpr (FMT == FMT_BF16) {
-        constexpr int D = 8;  // ring of k-steps
-        const int n_steps = K / 32;
+        // The contraction range is walked in pairs of MFMA steps (64 elements = one 128-byte
+        // line of a weight row): in a pair, lane group g takes elements 16g .. 16g+7 in the first
+        // step and 16g+8 .. 16g+15 in the second, so a lane's two 16-byte loads are adjacent and
+        // the four lane groups cover the whole line.  Ring of four pairs, loads issued three
+        // pairs (one and a half stages) ahead of their use; nothing touches a loaded value
+        // before the pair that consumes it.
+        constexpr int DP = 4;
+        const int n_pairs = K / 64;
         const uint8_t* a_ptr[R];
         const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int row = group * 64 + tile_row_in_group(r0 + r, q);
-            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 8 * g);
+            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 16 * g);
         }
-        u32x4 ar[D][R];
-        auto load_a = [&](int slot, int n) {
-            const bool live = n < n_steps;
-            const size_t off = live ? (size_t)n * 64 : 0;
+        u32x4 ar[DP][2][R];
+        auto load_a = [&](int slot, int pair) {
+            const size_t off = (size_t)(pair < n_pairs ? pair : 0) * 128;  // a padding pair re-reads pair 0 (unused)
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[r] + off);
-                ar[slot][r] = live ? v : u32x4{0u, 0u, 0u, 0u};
-            }
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    ar[slot][h][r] = *reinterpret_cast<const u32x4*>(a_ptr[r] + off + 16 * h);
         };
 #pragma unroll
-        for (int i = 0; i < D - 1; ++i) load_a(i, i);
+        for (int i = 0; i < DP - 1; ++i) load_a(i, i);
         __syncthreads();
         for (int s0 = 0; s0 < n_pad; s0 += 2) {
 #pragma unroll
             for (int ss = 0; ss < 2; ++ss) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int u = 4 * ss + j;
-                    load_a((u + D - 1) % D, 4 * (s0 + ss) + j + D - 1);
-                    u32x4 b[NT];
+                for (int pp = 0; pp < 2; ++pp) {
+                    const int u = 2 * ss + pp;  // ring slot of this pair
+                    const int pair = 2 * (s0 + ss) + pp;
+                    load_a((u + DP - 1) % DP, pair + DP - 1);
+                    __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three pairs ahead of their use
+                    const bool live = pair < n_pairs;   // wave-uniform
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) b[t] = b_frag(s0 + ss, j, t);
+                    for (int h = 0; h < 2; ++h) {
+                        u32x4 b[NT];
 #pragma unroll
-                    for (int r = 0; r < R; ++r)
+                        for (int t = 0; t < NT; ++t) b[t] = b_frag(s0 + ss, 2 * pp + h, t);
 #pragma unroll
-                        for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(ar[u][r], b[t], acc[r][t]);
+                        for (int r = 0; r < R; ++r) {
+                            const u32x4 av = live ? ar[u][h][r] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                            for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
+                        }
+                    }
                 }
                 __syncthreads();
             }
@@ -838,12 +851,8 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             dim3 grid(ceil_div(a.rows / 32, 10), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, a);
         } else if (a.waves_per_block == 1) {
-            if constexpr (FMT == FMT_MXFP4) {
-                dim3 grid(ceil_div(a.rows / 32, 12), a.max_tiles);
-                hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, a);
-            } else {
-                return MOE_ERR_FORMAT;
-            }
+            dim3 grid(ceil_div(a.rows / 32, 12), a.max_tiles);
+            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, a);
         } else if (a.waves_per_block == 8) {
             dim3 grid(ceil_div(units, 8), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_kernel<FMT, R, EPI, 8>), grid, dim3(512), 0, stream, a);
