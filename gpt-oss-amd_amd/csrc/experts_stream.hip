@@ -686,27 +686,31 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     const int n_quads = ceil_div(n_stages, 4);
     const int rem_groups = G & 3;
 
-    // activation staging: this wave moves k-step wave%4 of token tiles wave/4, wave/4 + WAVES/4, ...
-    const int step_w = wave & 3;
+    // activation staging, LDS image as in the producer/consumer kernel (token tile t at t*4096, row
+    // q at q*256, 16-byte chunk c at position c ^ q): this wave moves the four-row block wave%4
+    // (256 contiguous bytes per row, whole cache lines) of token tiles wave/4, wave/4 + WAVES/4, ...
+    const int blk_w = wave & 3;
     const int half_w = wave >> 2;
-    const int k_lane = 32 * g + 8 * step_w;  // lane group g owns MX block g of a stage
+    const int q_dma = 4 * blk_w + (lane >> 4);     // row of the token tile this lane moves
+    const int chunk_dma = (lane & 15) ^ q_dma;     // chunk of the stage it fetches
     const uint8_t* b_row[TS];
 #pragma unroll
     for (int i = 0; i < TS; ++i) {
-        const int idx = min((half_w + kStagers * i) * 16 + q, nrows - 1);
+        const int idx = min((half_w + kStagers * i) * 16 + q_dma, nrows - 1);
         const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
         b_row[i] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
     }
     auto issue_b = [&](int s) {
-        const int k = s * kStageElems + k_lane;
+        const int k = s * kStageElems + 8 * chunk_dma;
         const size_t off = (k < K) ? (size_t)k * 2 : 0;  // past the row: re-read its start (weights are 0 there)
-        uint8_t* dst = lds + (size_t)(s & 1) * kStageBytes + (size_t)(step_w * NTMAX + half_w) * 1024;
+        uint8_t* dst = lds + (size_t)(s & 1) * kStageBytes + (size_t)half_w * 4096 + blk_w * 1024;
 #pragma unroll
-        for (int i = 0; i < TS; ++i) dma16(b_row[i] + off, dst + i * kStagers * 1024);
+        for (int i = 0; i < TS; ++i) dma16(b_row[i] + off, dst + i * kStagers * 4096);
     };
-    const uint8_t* const lds_rd = lds + (size_t)lane * 16;
-    auto b_frag = [&](int s, int j, int t) {
-        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & 1) * kStageBytes + (j * NTMAX + t) * 1024);
+    const uint8_t* const lds_rd = lds + (size_t)q * 256;
+    auto b_frag = [&](int s, int j, int t) {  // lane group g owns MX block g of a stage: chunk 4g + j
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & 1) * kStageBytes + t * 4096 +
+                                               (((4 * g + j) ^ q) << 4));
     };
 
     if (!active) {
