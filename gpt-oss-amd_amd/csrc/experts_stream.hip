@@ -727,10 +727,14 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
 
     const size_t tile_bytes = (size_t)G * 256;
     const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
+    // wave-uniform bases (scalar registers) + per-lane 32-bit offsets that never change
     const uint8_t* const a_base = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride +
-                                  (size_t)unit * 4 * tile_bytes + (size_t)lane * 16;
-    const uint8_t* const s_base = a.w_scales + (size_t)e * a.s_expert_stride + (size_t)unit * 4 * stile_bytes +
-                                  (size_t)lane * 4;
+                                  (size_t)unit * 4 * tile_bytes;
+    const uint8_t* const s_base = a.w_scales + (size_t)e * a.s_expert_stride + (size_t)unit * 4 * stile_bytes;
+    const uint32_t voff_w = (uint32_t)lane * 16;
+    // ragged last stage: a lane group past the last MX block re-reads block 0 and gets scale 0
+    const uint32_t voff_w_ragged = (uint32_t)((g < rem_groups ? lane : q) * 16);
+    const uint32_t voff_s = (uint32_t)lane * 4;
     f32x4 acc[R][NT];
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -738,26 +742,31 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
         for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
     u32x4 araw[2][R];
     uint32_t sw_cur[R], sw_nxt[R];
+    // Nothing touches a loaded weight before the stage that consumes it (an instruction on it at
+    // load time would make the wave wait for the load right there): a stage or MX block that does
+    // not exist re-reads one that does and is multiplied by scale 0.
     auto load_a = [&](int slot, int s) {
-        const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
-        const size_t off = live ? (size_t)s * 1024 : 0;
+        const int su = s < n_stages ? s : 0;
+        const bool ragged = rem_groups != 0 && su == n_stages - 1;
+        const uint32_t vo = ragged ? voff_w_ragged : voff_w;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(a_base + r * tile_bytes + off);
-            araw[slot][r] = live ? v : u32x4{0u, 0u, 0u, 0u};
-        }
+        for (int r = 0; r < R; ++r)
+            araw[slot][r] = *reinterpret_cast<const u32x4*>(a_base + r * tile_bytes + (size_t)su * 1024 + vo);
     };
     auto load_scales = [&](uint32_t (&dst)[R], int quad) {
         const size_t off = (size_t)min(quad, n_quads - 1) * 256;
 #pragma unroll
-        for (int r = 0; r < R; ++r) dst[r] = *reinterpret_cast<const uint32_t*>(s_base + r * stile_bytes + off);
+        for (int r = 0; r < R; ++r)
+            dst[r] = *reinterpret_cast<const uint32_t*>(s_base + r * stile_bytes + off + voff_s);
     };
     auto do_stage = [&](int slot, int qpos, int s) {
         issue_b(s + 1);
         load_a(slot ^ 1, s + 1);
+        __builtin_amdgcn_sched_barrier(0);  // next stage's loads are issued here, before this stage's MFMAs
+        const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
         float sc[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32((sw_cur[r] >> (8 * qpos)) & 0xFFu);
+        for (int r = 0; r < R; ++r) sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * qpos)) & 0xFFu) : 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             u32x4 av[R];
