@@ -767,6 +767,7 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
         float sc[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * qpos)) & 0xFFu) : 0.0f;
+        u32x4 bq[2];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             u32x4 av[R];
@@ -776,14 +777,17 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
                 mxfp4_dword_to_bf16x8(araw[slot][r][j], sc[r], d);
                 av[r] = u32x4{d[0], d[1], d[2], d[3]};
             }
-            // activation operands are read from LDS two token tiles ahead of the MFMAs that use them
-            u32x4 bq[2];
-            bq[0] = b_frag(s, j, 0);
-            if constexpr (NT > 1) bq[1] = b_frag(s, j, 1);
+            // activation operands are read from LDS two token tiles ahead of the MFMAs that use
+            // them, across the k-steps of the stage (NT is even, so the buffer parity carries over)
+            if (j == 0) {
+                bq[0] = b_frag(s, 0, 0);
+                bq[1] = b_frag(s, 0, 1);
+            }
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const u32x4 b = bq[t & 1];
                 if (t + 2 < NT) bq[t & 1] = b_frag(s, j, t + 2);
+                else if (j + 1 < 4) bq[t & 1] = b_frag(s, j + 1, t + 2 - NT);
                 __builtin_amdgcn_sched_barrier(0);  // keep the read above ahead of the MFMAs below
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc[r][t] = mfma_16x16x32(av[r], b, acc[r][t]);
