@@ -389,11 +389,16 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     // MXFP4 (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of 32 rows each.
     // Blocks run in rounds of one per CU, so the cheaper choice is the one with the smaller
     // rounds x rows-per-block product; more rows per block also re-read the activations less.
+    const int kCUs = 256;  // MI355X
     auto pick_consumers = [&](int rows) {
-        const int kCUs = 256;  // MI355X
         const int cost10 = ceil_div(ceil_div(rows / 32, 10) * est_tiles, kCUs) * 10;
         const int cost12 = ceil_div(ceil_div(rows / 32, 12) * est_tiles, kCUs) * 12;
         return cost12 <= cost10 ? 1 : 0;
+    };
+    // one row block more than necessary when that makes the block count a whole number of rounds
+    auto pick_row_blocks = [&](int rows, int kernel) {
+        const int p = ceil_div(rows / 32, kernel == 1 ? 12 : 10);
+        return ((p * est_tiles) % kCUs != 0 && ((p + 1) * est_tiles) % kCUs == 0) ? p + 1 : p;
     };
     auto pick_kernel = [&](int rows) {
         return prefill ? 16 : pick_consumers(rows);
@@ -410,6 +415,7 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     a1.K = H;
     a1.bias_expert_stride = 2LL * I;
     a1.waves_per_block = pick_kernel(2 * I);
+    a1.row_blocks = prefill ? 0 : pick_row_blocks(2 * I, a1.waves_per_block);
     if (fmt == MOE_WEIGHTS_BF16) {
         a1.w_expert_stride = 2LL * I * H;
     } else {
@@ -434,6 +440,7 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     a2.K = I;
     a2.bias_expert_stride = H;
     a2.waves_per_block = pick_kernel(H);
+    a2.row_blocks = prefill ? 0 : pick_row_blocks(H, a2.waves_per_block);
     if (fmt == MOE_WEIGHTS_BF16) {
         a2.w_expert_stride = (long long)H * I;
     } else {

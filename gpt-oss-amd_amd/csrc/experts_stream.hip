@@ -606,8 +606,12 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
         else if (nt == 2) ws_producer<FMT, 2, PROD>(a, lds, row0, nrows, p);
         else ws_producer<FMT, 1, PROD>(a, lds, row0, nrows, p);
     } else {
-        const int unit = blockIdx.x * CONS + wave;
-        const bool active = unit < a.rows / 32;
+        // the row units of the weight matrix are spread evenly over the gridDim.x row blocks
+        const int units = a.rows / 32;
+        const int u0 = (int)((long long)blockIdx.x * units / gridDim.x);
+        const int u1 = (int)((long long)(blockIdx.x + 1) * units / gridDim.x);
+        const int unit = u0 + wave;
+        const bool active = unit < u1;
         if (nt == 4) ws_consumer<FMT, 4, EPI>(a, lds, e, row0, nrows, unit, active);
         else if (nt == 3) ws_consumer<FMT, 3, EPI>(a, lds, e, row0, nrows, unit, active);
         else if (nt == 2) ws_consumer<FMT, 2, EPI>(a, lds, e, row0, nrows, unit, active);
@@ -865,10 +869,10 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             dim3 grid(ceil_div(a.rows / 64, 8), a.max_tiles);
             hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 8>), grid, dim3(512), 0, stream, a);
         } else if (a.waves_per_block == 0) {
-            dim3 grid(ceil_div(a.rows / 32, 10), a.max_tiles);
+            dim3 grid(max(a.row_blocks, ceil_div(a.rows / 32, 10)), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, a);
         } else if (a.waves_per_block == 1) {
-            dim3 grid(ceil_div(a.rows / 32, 12), a.max_tiles);
+            dim3 grid(max(a.row_blocks, ceil_div(a.rows / 32, 12)), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, a);
         } else if (a.waves_per_block == 8) {
             dim3 grid(ceil_div(units, 8), a.max_tiles);

@@ -59,6 +59,7 @@ struct ExpertGemmArgs {
     float alpha, limit;
     int max_tiles;
     int format;
+    int row_blocks;             // producer-consumer kernel: row blocks per token block (0 = as few as fit)
     int waves_per_block;        // kernel choice: 0 / 1 producer-consumer kernel with 10 / 12 consumer waves (+ 2
                                 // producers); 8 or 4 uniform waves, 64-token blocks; 16 / 17 prefill kernel
                                 // (4 / 8 waves, 128-token blocks)
