@@ -212,10 +212,8 @@ def main():
     # the gate/up GEMM launch: which kernel serves it depends on bucket size and weight format
     if shape.T * shape.K >= 96 * shape.E:
         kname = "expert_prefill_kernel<%d, 0" % (0 if shape.fmt == "bf16" else 1)
-    elif shape.fmt == "bf16":
-        kname = "expert_stream_kernel<0, 2, 0"
     else:
-        kname = "expert_stream_ws_kernel<1, 0"
+        kname = "expert_stream_ws_kernel<%d, 0" % (0 if shape.fmt == "bf16" else 1)
     traffic = profiled_traffic(ge.ROOT, shape.name, kname)
     if bound == "hbm":
         achieved = head["mlp1"]["bytes"] / (head["mlp1"]["ms"] * 1e-3) / 1e9
