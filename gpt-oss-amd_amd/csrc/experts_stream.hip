@@ -43,18 +43,27 @@ MOE_DEVICE u32x4 pack_f32x8_to_bf16x8(const float4& lo, const float4& hi) {
 
 // Epilogue shared by the expert kernels: lane (q,g) of the 16x16 accumulator layout holds token
 // t*16+q and weight rows group*64 + g*16 + (r0+r)*4 + j (j = 0..3) for its R row tiles.
+// The four bias values per row tile of a lane; loaded before the main loop by the kernels that
+// want the load latency off the block's tail.
+template <int R>
+MOE_DEVICE void load_bias(const ExpertGemmArgs& a, int e, int group, int r0, uint2 (&raw)[R]) {
+    const int g = (threadIdx.x & 63) >> 4;
+    const uint16_t* bias = a.bias + (size_t)e * a.bias_expert_stride + group * 64 + g * 16 + r0 * 4;
+#pragma unroll
+    for (int r = 0; r < R; ++r) raw[r] = *reinterpret_cast<const uint2*>(bias + 4 * r);
+}
+
 template <int R, int NT, int EPI>
 MOE_DEVICE void stream_epilogue(const ExpertGemmArgs& a, const f32x4 (&acc)[R][NT], int e, int row0, int nrows,
-                                int group, int r0) {
+                                int group, int r0, const uint2 (&bias_raw)[R]) {
     const int lane = threadIdx.x & 63;
     const int q = lane & 15;
     const int g = lane >> 4;
     const int row_base = group * 64 + g * 16 + r0 * 4;
-    const uint16_t* bias = a.bias + (size_t)e * a.bias_expert_stride + row_base;
     float bv[R][4];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const uint2 raw = *reinterpret_cast<const uint2*>(bias + 4 * r);
+        const uint2 raw = bias_raw[r];
         bv[r][0] = bf16_bits_to_f32(raw.x & 0xFFFFu);
         bv[r][1] = bf16_bits_to_f32(raw.x >> 16);
         bv[r][2] = bf16_bits_to_f32(raw.y & 0xFFFFu);
@@ -337,7 +346,9 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
         }
     }
 
-    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0);
+    uint2 bias_raw[R];
+    load_bias<R>(a, e, group, r0, bias_raw);
+    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0, bias_raw);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -440,6 +451,8 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     }
     const int group = unit >> 1;
     const int r0 = (unit & 1) * R;
+    uint2 bias_raw[R];  // fetched now, used by the epilogue
+    load_bias<R>(a, e, group, r0, bias_raw);
     const uint8_t* const lds_rd = lds + (size_t)q * 256;
     auto b_frag = [&](int s, int j, int t) {
         return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes + t * 4096 +
@@ -584,7 +597,7 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
             for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
         }
     }
-    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0);
+    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0, bias_raw);
 }
 
 // grid = (ceil(row units / CONS), max_tiles), block = 64 (CONS + PROD); one block per CU: twelve
@@ -812,7 +825,9 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
 #pragma unroll
         for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
     }
-    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, unit, 0);
+    uint2 bias_raw[R];
+    load_bias<R>(a, e, unit, 0, bias_raw);
+    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, unit, 0, bias_raw);
 }
 
 template <int FMT, int NT, int EPI, int WAVES>
