@@ -398,7 +398,12 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
     const int sub = lane >> 4;   // row inside the instruction's block of four
     const int K = a.K;
     const int n_pad = ws_padded_stages<FMT>(K);
-    // this wave moves row blocks BP*p .. BP*p + BP-1 of every token tile
+    // this wave moves row blocks BP*p .. BP*p + BP-1 of every token tile; in the bucket's last token
+    // tile only those that hold a row of the bucket (n_last of them, the others stay stale in LDS:
+    // the accumulator columns they feed are never stored)
+    int n_last = 0;
+#pragma unroll
+    for (int ii = 0; ii < BP; ++ii) n_last += (16 * (NT - 1) + 4 * (BP * p + ii) < nrows) ? 1 : 0;
     const uint8_t* row[NT][BP];
     int chunk[BP];
 #pragma unroll
@@ -419,17 +424,25 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
             const int k = s * kStageElems + 8 * chunk[ii];
             const size_t off = (k < K) ? (size_t)k * 2 : 0;  // a position past the row re-reads its start
 #pragma unroll
-            for (int t = 0; t < NT; ++t) dma16(row[t][ii] + off, slot + t * 4096 + (BP * p + ii) * 1024);
+            for (int t = 0; t < NT; ++t)
+                if (t < NT - 1 || ii < n_last) dma16(row[t][ii] + off, slot + t * 4096 + (BP * p + ii) * 1024);
         }
+    };
+    // stage s has landed once only the loads of the two stages issued after it are outstanding
+    auto wait_two_stages = [&]() {
+        static_assert(BP == 2, "three possible load counts per stage");
+        if (n_last == 2) wait_vmcnt<2 * Q>();
+        else if (n_last == 1) wait_vmcnt<2 * Q - 2>();
+        else wait_vmcnt<2 * Q - 4>();
     };
     issue(0);
     issue(1);
     issue(2);
-    wait_vmcnt<2 * Q>();  // stage 0 has landed
+    wait_two_stages();  // stage 0 has landed
     __syncthreads();
     for (int i = 0; i < n_pad; ++i) {
         issue(i + 3);
-        wait_vmcnt<2 * Q>();  // stage i+1 has landed
+        wait_two_stages();  // stage i+1 has landed
         __syncthreads();
     }
     wait_vmcnt<0>();  // nothing may still be writing this block's LDS when the wave ends
