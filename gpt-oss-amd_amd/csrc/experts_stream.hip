@@ -18,6 +18,8 @@
 //   bf16  : elements 32j + 8g .. +8   (one 128-bit load per row tile and k-step)
 //   MXFP4 : elements 32g + 8j .. +8   (lane group g owns MX block g of the stage: one 128-bit load
 //           + one scale byte per row tile and stage, dequantised in registers to four A operands)
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -357,7 +359,7 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
 // activation rows global -> LDS with direct-to-LDS 128-bit loads (no registers, a ring of four
 // 16 KiB stage slots, three stages ahead of the consumers); consumers only have weight loads in
 // their memory queue.  One barrier per stage; every wave of the block executes exactly
-// 1 + n_pad barriers.
+// 1 + ceil(K / 128) barriers.
 // Positions of the contraction range that do not exist (ragged last stage, padding stages) carry
 // a weight operand of exact zeros; the activation operand there is a clamped re-read of real data.
 // ---------------------------------------------------------------------------------------------
@@ -373,11 +375,6 @@ MOE_DEVICE void dma16(const void* gsrc, uint8_t* lds_dst_wave_uniform) {
                                      (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 16, 0, 0);
 }
 
-template <int FMT>
-MOE_DEVICE int ws_padded_stages(int K) {
-    const int n_stages = ceil_div(K, kStageElems);
-    return (FMT == FMT_BF16) ? ceil_div(n_stages, 2) * 2 : ceil_div(n_stages, 4) * 4;
-}
 
 // LDS image of one stage of activations: token tile t at t*4096, row q (0..15) of the tile at
 // q*256, and inside the row the sixteen 16-byte chunks of the stage's 128 contraction elements,
@@ -397,7 +394,7 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
     const int pos = lane & 15;   // chunk position inside the row's LDS image
     const int sub = lane >> 4;   // row inside the instruction's block of four
     const int K = a.K;
-    const int n_pad = ws_padded_stages<FMT>(K);
+    const int n_stages = ceil_div(K, kStageElems);
     // this wave moves row blocks BP*p .. BP*p + BP-1 of every token tile; in the bucket's last token
     // tile only those that hold a row of the bucket (n_last of them, the others stay stale in LDS:
     // the accumulator columns they feed are never stored)
@@ -440,8 +437,8 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
     issue(2);
     wait_two_stages();  // stage 0 has landed
     __syncthreads();
-    for (int i = 0; i < n_pad; ++i) {
-        issue(i + 3);
+    for (int i = 0; i < n_stages; ++i) {
+        issue(i + 3);  // past the last stage: a re-read nobody consumes
         wait_two_stages();  // stage i+1 has landed
         __syncthreads();
     }
@@ -457,9 +454,8 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     const int q = lane & 15;
     const int K = a.K;
     const int n_stages = ceil_div(K, kStageElems);
-    const int n_pad = ws_padded_stages<FMT>(K);
     if (!active) {
-        for (int i = 0; i <= n_pad; ++i) __syncthreads();
+        for (int i = 0; i <= n_stages; ++i) __syncthreads();
         return;
     }
     const int group = unit >> 1;
@@ -505,32 +501,38 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
 #pragma unroll
         for (int i = 0; i < DP - 1; ++i) load_a(i, i);
         __syncthreads();
-        for (int s0 = 0; s0 < n_pad; s0 += 2) {
+        // one stage = two pairs; `ss` (stage parity) fixes the ring slots at compile time
+        auto stage = [&](auto ss_tag, int st) {
+            constexpr int ss = decltype(ss_tag)::value;
 #pragma unroll
-            for (int ss = 0; ss < 2; ++ss) {
+            for (int pp = 0; pp < 2; ++pp) {
+                constexpr int kSlots = DP;
+                const int u = 2 * ss + pp;  // ring slot of this pair
+                const int pair = 2 * st + pp;
+                load_a((u + kSlots - 1) % kSlots, pair + kSlots - 1);
+                __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three pairs ahead of their use
+                const bool live = pair < n_pairs;   // wave-uniform; false only in the second half of a ragged stage
 #pragma unroll
-                for (int pp = 0; pp < 2; ++pp) {
-                    const int u = 2 * ss + pp;  // ring slot of this pair
-                    const int pair = 2 * (s0 + ss) + pp;
-                    load_a((u + DP - 1) % DP, pair + DP - 1);
-                    __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three pairs ahead of their use
-                    const bool live = pair < n_pairs;   // wave-uniform
+                for (int h = 0; h < 2; ++h) {
+                    u32x4 b[NT];
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        u32x4 b[NT];
+                    for (int t = 0; t < NT; ++t) b[t] = b_frag(st, 2 * pp + h, t);
 #pragma unroll
-                        for (int t = 0; t < NT; ++t) b[t] = b_frag(s0 + ss, 2 * pp + h, t);
+                    for (int r = 0; r < R; ++r) {
+                        const u32x4 av = live ? ar[u][h][r] : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-                        for (int r = 0; r < R; ++r) {
-                            const u32x4 av = live ? ar[u][h][r] : u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-                            for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
-                        }
+                        for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
                     }
                 }
-                __syncthreads();
             }
+            __syncthreads();
+        };
+        const int n_even = n_stages & ~1;
+        for (int s0 = 0; s0 < n_even; s0 += 2) {
+            stage(std::integral_constant<int, 0>{}, s0);
+            stage(std::integral_constant<int, 1>{}, s0 + 1);
         }
+        if (n_stages & 1) stage(std::integral_constant<int, 0>{}, n_even);
     } else {
         // Weights: a ring of four stages (one 128-bit load per row tile and stage, issued three
         // stages ahead of its use); scales: one word per row tile covers four stages and is
@@ -541,7 +543,6 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         constexpr int D = 4;
         const int G = K / 32;
         const int rem_groups = G & 3;  // MX blocks in a ragged last stage (0 = none)
-        const int n_quads = n_pad / 4;
         const size_t tile_bytes = (size_t)G * 256;
         const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
         const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
@@ -578,37 +579,46 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
 #pragma unroll
         for (int i = 0; i < D - 1; ++i) load_a(i, i);
         __syncthreads();
-        for (int qd = 0; qd < n_quads; ++qd) {
-            load_scales(sw_nxt, qd + 1);
+        // stage st, the i-th of its group of four (i fixes ring slot and scale byte at compile time)
+        auto stage = [&](auto i_tag, int st) {
+            constexpr int i = decltype(i_tag)::value;
+            load_a((i + D - 1) % D, st + D - 1);
+            __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three stages ahead of their use
+            const bool live = !(rem_groups != 0 && st == n_stages - 1 && g >= rem_groups);
+            float sc[R];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int s = 4 * qd + i;
-                load_a((i + D - 1) % D, s + D - 1);
-                __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three stages ahead of their use
-                const bool live = s < n_stages && !(rem_groups != 0 && s == n_stages - 1 && g >= rem_groups);
-                float sc[R];
+            for (int r = 0; r < R; ++r) sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu) : 0.0f;
 #pragma unroll
-                for (int r = 0; r < R; ++r)
-                    sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu) : 0.0f;
+            for (int j = 0; j < 4; ++j) {
+                u32x4 b[NT];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    u32x4 b[NT];
+                for (int t = 0; t < NT; ++t) b[t] = b_frag(st, j, t);
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) b[t] = b_frag(s, j, t);
+                for (int r = 0; r < R; ++r) {
+                    uint32_t d[4];
+                    mxfp4_dword_to_bf16x8(araw[i][r][j], sc[r], d);
+                    const u32x4 av = {d[0], d[1], d[2], d[3]};
 #pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        uint32_t d[4];
-                        mxfp4_dword_to_bf16x8(araw[i][r][j], sc[r], d);
-                        const u32x4 av = {d[0], d[1], d[2], d[3]};
-#pragma unroll
-                        for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
-                    }
+                    for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
                 }
-                __syncthreads();
             }
+            __syncthreads();
+        };
+        const int full_quads = n_stages / 4;
+        for (int qd = 0; qd < full_quads; ++qd) {
+            load_scales(sw_nxt, qd + 1);
+            stage(std::integral_constant<int, 0>{}, 4 * qd + 0);
+            stage(std::integral_constant<int, 1>{}, 4 * qd + 1);
+            stage(std::integral_constant<int, 2>{}, 4 * qd + 2);
+            stage(std::integral_constant<int, 3>{}, 4 * qd + 3);
 #pragma unroll
             for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
         }
+        // the last, partial group of four (wave-uniform conditions; its weights are already in the ring)
+        const int tail = n_stages - 4 * full_quads;
+        if (tail > 0) stage(std::integral_constant<int, 0>{}, 4 * full_quads + 0);
+        if (tail > 1) stage(std::integral_constant<int, 1>{}, 4 * full_quads + 1);
+        if (tail > 2) stage(std::integral_constant<int, 2>{}, 4 * full_quads + 2);
     }
     stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0, bias_raw);
 }
@@ -747,7 +757,7 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
         issue_b(0);
         wait_vmcnt<0>();
         __syncthreads();
-        for (int s = 0; s < 4 * n_quads; ++s) {
+        for (int s = 0; s < n_stages; ++s) {
             issue_b(s + 1);
             wait_vmcnt<0>();
             __syncthreads();
@@ -834,7 +844,8 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     for (int qd = 0; qd < n_quads; ++qd) {
         load_scales(sw_nxt, qd + 1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) do_stage(i & 1, i, 4 * qd + i);
+        for (int i = 0; i < 4; ++i)
+            if (4 * qd + i < n_stages) do_stage(i & 1, i, 4 * qd + i);  // block-uniform: the last group may be partial
 #pragma unroll
         for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
     }
