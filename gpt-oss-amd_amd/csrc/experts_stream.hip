@@ -432,15 +432,19 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
         else if (n_last == 1) wait_vmcnt<2 * Q - 2>();
         else wait_vmcnt<2 * Q - 4>();
     };
+    // Bare s_barrier, not __syncthreads(): the fence of __syncthreads() makes the compiler wait for
+    // every outstanding direct-to-LDS load (vmcnt(0)) in front of each barrier, i.e. also for the
+    // stages issued just now, and the ring would hide nothing.  The explicit wait above each barrier
+    // is the guarantee the consumers need: the stage they read next has been written to LDS.
     issue(0);
     issue(1);
     issue(2);
     wait_two_stages();  // stage 0 has landed
-    __syncthreads();
+    __builtin_amdgcn_s_barrier();
     for (int i = 0; i < n_stages; ++i) {
         issue(i + 3);  // past the last stage: a re-read nobody consumes
         wait_two_stages();  // stage i+1 has landed
-        __syncthreads();
+        __builtin_amdgcn_s_barrier();
     }
     wait_vmcnt<0>();  // nothing may still be writing this block's LDS when the wave ends
 }
