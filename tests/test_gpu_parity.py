@@ -175,6 +175,8 @@ SMALL = [
     (300, 128, 64, 4, 4, "mxfp4"),       # every token uses every expert: 300 rows per expert, 5 token blocks
     (33, 192, 64, 128, 4, "bf16"),       # most experts empty
     (17, 2880, 2880, 4, 2, "mxfp4"),     # real row/contraction lengths, few experts
+    (64, 512, 256, 8, 4, "mxfp4"),       # contraction lengths that are whole groups of four stages / two stages
+    (64, 512, 256, 8, 4, "bf16"),
     # prefill-sized buckets (T*K >= 96*E): 128-token blocks, every token-tile count from 1 to 8
     (300, 128, 64, 4, 4, "bf16"),
     (700, 320, 192, 8, 4, "mxfp4"),      # ragged last MX chunk on the gate/up side
