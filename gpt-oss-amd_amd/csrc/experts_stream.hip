@@ -1,23 +1,29 @@
-// Weight-streaming expert GEMM for decode-sized buckets (tens of rows per expert).
-//
-// Every weight byte is loaded from HBM exactly once per token block, straight into the MFMA
-// A-operand registers with 128-bit loads (no LDS for weights: a weight element is used by one wave
-// only).  The bucket's activation rows are the B operand; the four waves of a block share them
-// through LDS, staged 128 contraction elements at a time in MFMA operand order (one contiguous
-// KiB per k-step and token tile, so the 128-bit LDS reads are conflict-free), double-buffered so
-// one barrier per stage suffices.  fp32 accumulation in v_mfma_f32_16x16x32_bf16.
+// Expert GEMMs of the MoE block: y = W x + b per expert over its bucket of token rows, with the
+// SwiGLU (gate/up launch) or the per-slot row store (down launch) in the epilogue.
 // Replaces moe_mlp1_swiglu_mfma_kernel (src/hip/moe.hip:9-235) and moe_mlp2_scatter_mfma_kernel
-// (src/hip/moe.hip:261-512) for small buckets; the arithmetic contract is the CPU path's
-// (src/run.cpp:657-705): y = W x + b, SwiGLU on interleaved gate/up rows, down projection.
+// (src/hip/moe.hip:261-512); the arithmetic contract is the CPU path's (src/run.cpp:657-705).
 //
-// Work split: block (x = group of row units, y = token block).  A block has 4 waves; each wave
-// owns R MFMA row tiles (16R weight rows) over the whole contraction length and up to NT*16 tokens.
+// Common to all kernels here: every weight byte is loaded from HBM once per token block, straight
+// into the MFMA A-operand registers with 128-bit loads (no LDS for weights: a weight element is
+// used by one wave only); the bucket's activation rows are the B operand and are shared by the
+// waves of a block through LDS, 128 contraction elements (one stage) at a time, one barrier per
+// stage; fp32 accumulation in v_mfma_f32_16x16x32_bf16.  A wave owns R MFMA row tiles (16 R weight
+// rows) over the whole contraction length and up to NT*16 tokens.
+//
 // The contraction index is a dummy index, so lanes are free to pick which k each of their eight
-// operand elements stands for as long as A and B agree.  Inside a stage of 128 elements, k-step j
-// (0..3) and lane group g = lane/16 take
-//   bf16  : elements 32j + 8g .. +8   (one 128-bit load per row tile and k-step)
-//   MXFP4 : elements 32g + 8j .. +8   (lane group g owns MX block g of the stage: one 128-bit load
-//           + one scale byte per row tile and stage, dequantised in registers to four A operands)
+// operand elements stands for as long as A and B agree.  Inside a stage, k-step j (0..3) and lane
+// group g = lane/16 take
+//   bf16, uniform-wave kernel    : elements 32j + 8g .. +8
+//   bf16, producer/consumer      : elements 64(j/2) + 16g + 8(j%2) .. +8  (a lane's two loads of a
+//                                  pair of steps are adjacent: whole 128-byte lines per row)
+//   MXFP4                        : elements 32g + 8j .. +8  (lane group g owns MX block g of the
+//                                  stage: one 128-bit load + one scale byte per row tile and stage,
+//                                  dequantised in registers to four A operands)
+//
+// Kernels: expert_stream_ws_kernel (decode-sized buckets, producer and consumer waves, the one the
+// fused block uses), expert_stream_kernel / expert_stream_queue_kernel (uniform waves, activations
+// staged through registers; serve the reference-signature entries), expert_prefill_kernel
+// (128-token blocks, 64 x 128 tile per wave).
 #include <type_traits>
 
 #include "common.h"
