@@ -578,7 +578,12 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
             const uint32_t vo = ragged ? voff_w_ragged : voff_w;
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                araw[slot][r] = *reinterpret_cast<const u32x4*>(wtile[r] + (size_t)su * 1024 + vo);
+                // non-temporal: a 1 KiB chunk is read once, by this instruction alone, so keeping its
+                // lines in L1/L2 only evicts the activation rows (measured: -5 % kernel time; the bf16
+                // path, where two instructions share each line, and the prefill kernel, where
+                // neighbouring token blocks re-read the weights, are slower with it)
+                araw[slot][r] =
+                    __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wtile[r] + (size_t)su * 1024 + vo));
         };
         auto load_scales = [&](uint32_t (&dst)[R], int quad) {
             const size_t off = (size_t)min(quad, last_quad) * 256;
