@@ -1,5 +1,6 @@
 // extern "C" entry points of libmoe_gfx950.so (declared in include/moe_abi.h): argument checks,
 // workspace carving and launch sequencing.  No entry allocates, synchronises or exits.
+#include "../../include/moe_checkpoint.h"
 #include "common.h"
 #include "kernels.h"
 
@@ -92,6 +93,9 @@ const char* moe_error_string(int code) {
         case MOE_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case MOE_ERR_FORMAT: return "unknown weight format or flag";
         case MOE_ERR_ALIGN: return "a pointer does not have the documented alignment";
+        case MOE_ERR_IO: return "the file cannot be opened, sized or mapped";
+        case MOE_ERR_PARSE: return "malformed checkpoint header";
+        case MOE_ERR_MISSING: return "a tensor the call needs is not in the file";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }

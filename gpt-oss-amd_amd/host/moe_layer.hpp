@@ -8,6 +8,7 @@
 #include <cstdint>
 
 #include "../../include/moe_abi.h"
+#include "../../include/moe_checkpoint.h"
 
 namespace moe_host {
 
@@ -52,6 +53,52 @@ struct OssMoeRunState {
     void* workspace;      // moe_block_workspace_bytes(batch_size, ...), 256-byte aligned
     size_t workspace_bytes;
 };
+
+// Config of an open checkpoint (src/run.cpp:26-46) reduced to the MoE members.
+inline int moe_config_from_checkpoint(const moe_ckpt* ck, int batch_size, OssMoeConfig* out) {
+    moe_ckpt_config c;
+    const int rc = moe_ckpt_get_config(ck, &c);
+    if (rc) return rc;
+    *out = OssMoeConfig{c.hidden_dim,  c.n_experts,    c.experts_per_token, c.intermediate_dim,
+                        c.n_layers,    c.swiglu_limit, batch_size};
+    return MOE_OK;
+}
+
+// Fills the stacked device tensors of `w` (the caller allocated them, sized for every layer) from an
+// open checkpoint, layer by layer: the MoE part of copy_transformer_to_device (src/model.cpp:363-460).
+// MXFP4 files go to the w_mlp*_blocks / w_mlp*_scales members, dense files to w_mlp1 / w_mlp2.
+inline int moe_upload_weights(const moe_ckpt* ck, const OssMoeConfig& p, const OssMoeWeights& w, void* d_staging,
+                              size_t staging_bytes, moe_stream_t stream) {
+    const long long H = p.hidden_dim, I = p.intermediate_dim, E = p.n_experts;
+    const bool tiled = w.w_mlp1_blocks != nullptr;
+    size_t b1 = 0, s1 = 0, b2 = 0, s2 = 0;
+    if (tiled) {
+        moe_mxfp4_tiled_bytes(2 * p.intermediate_dim, p.hidden_dim, &b1, &s1);
+        moe_mxfp4_tiled_bytes(p.hidden_dim, p.intermediate_dim, &b2, &s2);
+    }
+    for (int l = 0; l < p.n_layers; ++l) {
+        moe_layer_device d{};
+        d.struct_bytes = sizeof(d);
+        d.weight_format = tiled ? MOE_WEIGHTS_MXFP4_TILED : MOE_WEIGHTS_BF16;
+        d.rms_ffn_w = const_cast<moe_bf16_t*>(w.rms_ffn_w) + l * H;
+        d.w_router = const_cast<moe_bf16_t*>(w.w_router) + l * E * H;
+        d.b_router = const_cast<moe_bf16_t*>(w.b_router) + l * E;
+        d.b_mlp1 = const_cast<moe_bf16_t*>(w.b_mlp1) + l * E * 2 * I;
+        d.b_mlp2 = const_cast<moe_bf16_t*>(w.b_mlp2) + l * E * H;
+        if (tiled) {
+            d.w_mlp1 = const_cast<uint8_t*>(w.w_mlp1_blocks) + (size_t)l * E * b1;
+            d.w_mlp1_scales = const_cast<uint8_t*>(w.w_mlp1_scales) + (size_t)l * E * s1;
+            d.w_mlp2 = const_cast<uint8_t*>(w.w_mlp2_blocks) + (size_t)l * E * b2;
+            d.w_mlp2_scales = const_cast<uint8_t*>(w.w_mlp2_scales) + (size_t)l * E * s2;
+        } else {
+            d.w_mlp1 = const_cast<moe_bf16_t*>(w.w_mlp1) + l * E * 2 * I * H;
+            d.w_mlp2 = const_cast<moe_bf16_t*>(w.w_mlp2) + l * E * H * I;
+        }
+        const int rc = moe_ckpt_upload_layer(ck, l, &d, d_staging, staging_bytes, stream);
+        if (rc) return rc;
+    }
+    return MOE_OK;
+}
 
 inline size_t moe_workspace_bytes(const OssMoeConfig& p) {
     return moe_block_workspace_bytes(p.batch_size, p.hidden_dim, p.intermediate_dim, p.n_experts, p.experts_per_token);

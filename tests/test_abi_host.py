@@ -127,3 +127,14 @@ def test_cpp_host_headers_compile_link_and_check_arguments(pkg, tmp_path):
     r = subprocess.run([exe], capture_output=True, text=True)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "workspace for B=256" in r.stdout
+    # the same program describes a checkpoint file in either on-disk format
+    import ckptgen
+    tensors = ckptgen.make_tensors(ckptgen.TINY, seed=1, mxfp4=False)
+    ckptgen.write_bin(tmp_path / "m.bin", ckptgen.TINY, tensors)
+    r = subprocess.run([exe, str(tmp_path / "m.bin")], capture_output=True, text=True)
+    assert r.returncode == 0 and "3 layers, 4 experts, H=64, I=32, dense experts" in r.stdout, r.stdout
+    ckptgen.write_safetensors(tmp_path / "m.safetensors", ckptgen.make_tensors(ckptgen.TINY, seed=1, mxfp4=True))
+    r = subprocess.run([exe, str(tmp_path / "m.safetensors")], capture_output=True, text=True)
+    assert r.returncode == 0 and "MXFP4 experts" in r.stdout, r.stdout
+    r = subprocess.run([exe, str(tmp_path / "absent.bin")], capture_output=True, text=True)
+    assert r.returncode == 2 and "cannot be opened" in r.stdout
