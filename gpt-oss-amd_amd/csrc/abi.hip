@@ -52,7 +52,8 @@ struct BlockWorkspace {
             return p;
         };
         const int S = router_segments(T, E, H, false);
-        router_partial = static_cast<double*>(take((size_t)S * T * E * sizeof(double)));
+        router_partial = static_cast<double*>(
+            take(std::max((size_t)S * T * E * sizeof(double), router_two_pass(T, E, H) ? router_screen_bytes(T, E, H) : 0)));
         t_bf16 = static_cast<uint16_t*>(take((size_t)T * H * 2));
         expert_offsets = static_cast<int*>(take((size_t)(E + 1) * 4));
         tokens_flat = static_cast<int*>(take(A * 4));
@@ -354,13 +355,22 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     if ((rc = mark())) return rc;
 
     // 1. router logits -> top-k -> softmax  (src/forward.cpp:318-327; src/run.cpp:630-642)
-    const int S = router_segments(T, E, H, (p->flags & MOE_FLAG_ROUTER_STRICT_ORDER) != 0);
-    rc = launch_router_partial(p->t, p->w_router, ws.router_partial, ws.t_bf16, T, H, E, S, stream);
-    if (rc) return rc;
-    if ((rc = mark())) return rc;
-    rc = launch_router_finalize(ws.router_partial, S, nullptr, p->b_router, p->router_score, p->topk_v, p->topk_i, T, E,
-                                K, 1, 1, stream);
-    if (rc) return rc;
+    // Large batches without a request for the full score matrix take the two-pass router (same
+    // indices and weights); everything else the single exact pass.
+    const bool strict = (p->flags & MOE_FLAG_ROUTER_STRICT_ORDER) != 0;
+    if (!strict && !p->router_score && router_two_pass(T, E, H)) {
+        rc = launch_router_two_pass(p->t, p->w_router, p->b_router, ws.router_partial, ws.t_bf16, p->topk_v, p->topk_i, T,
+                                    H, E, K, 1, stream, timer ? timer->ev[stage++] : nullptr);
+        if (rc) return rc;
+    } else {
+        const int S = router_segments(T, E, H, strict);
+        rc = launch_router_partial(p->t, p->w_router, ws.router_partial, ws.t_bf16, T, H, E, S, stream);
+        if (rc) return rc;
+        if ((rc = mark())) return rc;
+        rc = launch_router_finalize(ws.router_partial, S, nullptr, p->b_router, p->router_score, p->topk_v, p->topk_i, T,
+                                    E, K, 1, 1, stream);
+        if (rc) return rc;
+    }
     if ((rc = mark())) return rc;
 
     // 2. bucketing + token-block map  (src/forward.cpp:329-376)
@@ -387,7 +397,6 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
 
     // eight waves (256 weight rows) per block when that still yields enough blocks to fill the chip
     const int est_tiles = std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
-    auto pick_waves = [&](int rows) { return ceil_div(rows / 32, 8) * est_tiles >= 512 ? 8 : 4; };
     // measured on MI355X at decode shapes: bf16 weights stream fastest with uniform waves, MXFP4
     // weights (four times the work per byte) with producer/consumer waves
     // MXFP4 (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of 32 rows each.

@@ -95,6 +95,57 @@ MOE_DEVICE f32x16 mfma_32x32x16(const u32x4& a, const u32x4& b, f32x16 c) {
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// ---- wave-wide reductions on the DPP path -----------------------------------------------------
+// Six data-parallel-primitive steps (shift right by 1, 2, 4, 8 inside each row of 16 lanes, then
+// the two row broadcasts) leave the combination of all 64 lanes in lane 63; a lane whose source
+// falls outside its row keeps `identity`.  No LDS traffic and no waiting on the LDS queue, unlike
+// the ds_bpermute behind __shfl_xor.  The result is read from lane 63 into a scalar register, so
+// every lane gets it.
+template <int CTRL, int ROW_MASK>
+MOE_DEVICE uint32_t dpp_move(uint32_t identity, uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)identity, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+#define MOE_DPP_STEPS(STEP) \
+    STEP(0x111, 0xf)        \
+    STEP(0x112, 0xf)        \
+    STEP(0x114, 0xf)        \
+    STEP(0x118, 0xf)        \
+    STEP(0x142, 0xa)        \
+    STEP(0x143, 0xc)
+
+MOE_DEVICE float wave_sum(float v) {
+#define MOE_STEP(C, M) v += __uint_as_float(dpp_move<C, M>(0u, __float_as_uint(v)));
+    MOE_DPP_STEPS(MOE_STEP)
+#undef MOE_STEP
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
+}
+
+// for v >= 0
+MOE_DEVICE float wave_max_nonneg(float v) {
+#define MOE_STEP(C, M) v = fmaxf(v, __uint_as_float(dpp_move<C, M>(0u, __float_as_uint(v))));
+    MOE_DPP_STEPS(MOE_STEP)
+#undef MOE_STEP
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
+}
+
+// Fixed combination order (a pure function of the lane values), so results are reproducible.
+MOE_DEVICE double wave_sum(double v) {
+#define MOE_STEP(C, M)                                                          \
+    {                                                                           \
+        const uint64_t b = __builtin_bit_cast(uint64_t, v);                     \
+        const uint32_t lo = dpp_move<C, M>(0u, (uint32_t)b);                    \
+        const uint32_t hi = dpp_move<C, M>(0u, (uint32_t)(b >> 32));            \
+        v += __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);             \
+    }
+    MOE_DPP_STEPS(MOE_STEP)
+#undef MOE_STEP
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)b, 63);
+    const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(b >> 32), 63);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+
 // ---- clamped SwiGLU (src/run.cpp:673-689) ---------------------------------------------------
 MOE_DEVICE float swiglu(float gate, float up, float alpha, float limit) {
     gate = gate > limit ? limit : gate;

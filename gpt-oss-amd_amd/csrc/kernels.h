@@ -14,6 +14,14 @@ int launch_router_finalize(const double* partial, int S, const float* scores_in,
                            float* scores_out, float* topk_v, int* topk_i, int T, int E, int K, int do_topk,
                            int do_softmax, hipStream_t stream);
 int launch_softmax_rows(float* x, int B, int size, hipStream_t stream);
+// Two-pass router (fp32 screening of all experts, exact scores of the candidates): same top-k and
+// softmax as partial + finalize.  `scratch` holds router_screen_bytes(); `between`, if not NULL, is
+// recorded after the first pass.
+bool router_two_pass(int T, int E, int H);
+size_t router_screen_bytes(int T, int E, int H);
+int launch_router_two_pass(const float* x, const uint16_t* w, const uint16_t* bias, void* scratch, uint16_t* x_bf16,
+                           float* topk_v, int* topk_i, int T, int H, int E, int K, int do_softmax,
+                           hipStream_t stream, hipEvent_t between);
 
 // ---- bucket.hip -------------------------------------------------------------------------------
 // Token-block map consumed by the expert kernels: tile i covers rows

@@ -132,6 +132,7 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const float* __rest
 // ---------------------------------------------------------------------------------------------
 constexpr int kSmallSeg = 192;
 
+
 __global__ __launch_bounds__(256) void router_partial_small_kernel(const float* __restrict__ x,
                                                                    const uint16_t* __restrict__ w,
                                                                    double* __restrict__ partial,
@@ -229,6 +230,77 @@ __global__ __launch_bounds__(256) void router_partial_small_kernel(const float* 
 // ---------------------------------------------------------------------------------------------
 MOE_DEVICE bool better(float va, int ia, float vb, int ib) { return va > vb || (va == vb && ia < ib); }
 
+// These kernels run their code once per wave, so their time is instruction fetch as much as
+// anything: loops stay rolled (the round and segment counts are wave-uniform anyway).
+//
+// K rounds of wave-wide argmax over vals[0..E) ordered by (value desc, index asc).  Lane r < K
+// ends up holding the winner of round r in (my_v, my_i).
+MOE_DEVICE void select_topk(const float* vals, int E, int K, int lane, float& my_v, int& my_i) {
+    uint32_t taken = 0;  // bit c set: candidate lane + 64*c already selected
+    my_v = -INFINITY;
+    my_i = 0;
+#pragma nounroll
+    for (int r = 0; r < K; ++r) {
+        float bv = -INFINITY;
+        int bi = 0x7FFFFFFF;
+#pragma nounroll
+        for (int c = 0, e = lane; e < E; ++c, e += 64) {
+            const float v = vals[e];
+            if (!(taken & (1u << c)) && (bi == 0x7FFFFFFF || better(v, e, bv, bi))) {
+                bv = v;
+                bi = e;
+            }
+        }
+        // wave-wide winner on the DPP path; a lane without a source keeps (any, 0x7FFFFFFF)
+#define MOE_STEP(C, M)                                                                      \
+    {                                                                                       \
+        const float ov = __uint_as_float(dpp_move<C, M>(0u, __float_as_uint(bv)));          \
+        const int oi = (int)dpp_move<C, M>(0x7FFFFFFFu, (uint32_t)bi);                      \
+        const bool take = oi != 0x7FFFFFFF && (bi == 0x7FFFFFFF || better(ov, oi, bv, bi)); \
+        bv = take ? ov : bv;                                                                \
+        bi = take ? oi : bi;                                                                \
+    }
+        MOE_DPP_STEPS(MOE_STEP)
+#undef MOE_STEP
+        bv = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(bv), 63));
+        bi = __builtin_amdgcn_readlane(bi, 63);
+        if (lane == r) {
+            my_v = bv;
+            my_i = bi;
+        }
+        if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
+    }
+}
+
+MOE_DEVICE float lane_value(float v, int src_lane) {
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), src_lane));
+}
+
+// Softmax of src/run.cpp:321-339 over the K selected values in its own order of operations (max,
+// then exponentials, then their fp64 sum in index order), or the values themselves; lane r < K
+// stores entry r.
+MOE_DEVICE void write_topk(float my_v, int my_i, int K, int lane, int do_softmax, float* __restrict__ out_v,
+                           int* __restrict__ out_i) {
+    float o = my_v;
+    if (do_softmax) {
+        double max_val = lane_value(my_v, 0);
+#pragma nounroll
+        for (int r = 1; r < K; ++r) {
+            const float v = lane_value(my_v, r);
+            if (v > max_val) max_val = v;
+        }
+        const float ex = expf((float)((double)my_v - max_val));
+        double sum = 0.0;
+#pragma nounroll
+        for (int r = 0; r < K; ++r) sum += (double)lane_value(ex, r);
+        o = (float)((double)ex / sum);
+    }
+    if (lane < K) {
+        out_v[lane] = o;
+        out_i[lane] = my_i;
+    }
+}
+
 __global__ __launch_bounds__(256) void router_finalize_kernel(const double* __restrict__ partial, int S,
                                                               const float* __restrict__ scores_in,
                                                               const uint16_t* __restrict__ bias,
@@ -246,14 +318,10 @@ __global__ __launch_bounds__(256) void router_finalize_kernel(const double* __re
     for (int e = lane; e < E; e += 64) {
         float v;
         if (partial) {
-            // all segment partials in flight at once, then summed in segment order
-            double part[16];
-#pragma unroll
-            for (int s = 0; s < 16; ++s) part[s] = s < S ? partial[((size_t)s * T + t) * E + e] : 0.0;
+            // summed in segment order; four loads in flight
             double sum = 0.0;
-#pragma unroll
-            for (int s = 0; s < 16; ++s)
-                if (s < S) sum += part[s];
+#pragma unroll 4
+            for (int s = 0; s < S; ++s) sum += partial[((size_t)s * T + t) * E + e];
             v = (float)sum;
             v += bf16_bits_to_f32(bias[e]);
         } else {
@@ -265,69 +333,233 @@ __global__ __launch_bounds__(256) void router_finalize_kernel(const double* __re
     if (!do_topk) return;
     __builtin_amdgcn_wave_barrier();
 
-    uint32_t taken = 0;  // bit c set: candidate lane + 64*c already selected
-    float sel_v[8];
-    int sel_i[8];
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-        sel_v[r] = 0.f;
-        sel_i[r] = 0;
-    }
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-        if (r < K) {
-            float bv = -INFINITY;
-            int bi = 0x7FFFFFFF;
-            for (int c = 0, e = lane; e < E; ++c, e += 64) {
-                if (taken & (1u << c)) continue;
-                const float v = my[e];
-                if (bi == 0x7FFFFFFF || better(v, e, bv, bi)) {
-                    bv = v;
-                    bi = e;
-                }
+    float my_v;
+    int my_i;
+    select_topk(my, E, K, lane, my_v, my_i);
+    write_topk(my_v, my_i, K, lane, do_softmax, topk_v + (size_t)t * K, topk_i + (size_t)t * K);
+}
+
+// ---------------------------------------------------------------------------------------------
+// First pass of the two-pass router: approximate logits of ALL experts on the matrix cores.
+// Every activation is split into two bf16 pieces, x = hi + lo + r with |r| <= 2^-16 |x|, and both
+// pieces are multiplied with the bf16 router weights (products of two bf16 are exact in fp32) and
+// accumulated in fp32 by v_mfma_f32_16x16x32_bf16.  Taking every fp32 addition inside the matrix
+// unit and every accumulation to be good to one unit in the last place, a partial over a segment
+// of n k-steps is within (33 + 2n) * 2^-23 * sum|w_k x_k| of the products it adds up.
+// A wave owns 16 tokens (MFMA rows) and NE tiles of 16 experts (MFMA columns) over one k-segment.
+// The same pass writes the bf16 copy of the activations (the hi pieces) for the expert GEMMs, the
+// squared norm of every token's segment (xn2 [S][T]) and, in the blocks of the first token tile,
+// of every router row's segment (wn2 [S][E]).  partial is [S][T][E] fp32.
+// grid = (ceil(T/64), ceil(E/(16*NE)), S), block = 256; seg_len % 32 == 0, H % 32 == 0.
+// ---------------------------------------------------------------------------------------------
+template <int NE>
+__global__ __launch_bounds__(256) void router_screen_kernel(const float* __restrict__ x,
+                                                            const uint16_t* __restrict__ w,
+                                                            float* __restrict__ partial, float* __restrict__ wn2,
+                                                            float* __restrict__ xn2, uint16_t* __restrict__ x_bf16,
+                                                            int T, int H, int E, int seg_len) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int t0 = blockIdx.x * 64 + wave * 16;
+    const int e_base = blockIdx.y * 16 * NE;
+    const int s = blockIdx.z;
+    const int kbeg = s * seg_len;
+    const int kend = min(H, kbeg + seg_len);
+    const bool first_group = blockIdx.y == 0;
+
+    if (blockIdx.x == 0) {  // block-uniform: squared norms of this block's router rows
+        for (int i = wave; i < 16 * NE; i += 4) {
+            const int e = e_base + i;
+            if (e >= E) break;
+            float q = 0.f;
+            for (int k = kbeg + lane; k < kend; k += 64) {
+                const float wf = bf16_bits_to_f32(w[(size_t)e * H + k]);
+                q = fmaf(wf, wf, q);
             }
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) {
-                const float ov = __shfl_xor(bv, off, 64);
-                const int oi = __shfl_xor(bi, off, 64);
-                if (oi != 0x7FFFFFFF && (bi == 0x7FFFFFFF || better(ov, oi, bv, bi))) {
-                    bv = ov;
-                    bi = oi;
-                }
-            }
-            sel_v[r] = bv;
-            sel_i[r] = bi;
-            if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
+            q = wave_sum(q);
+            if (lane == 0) wn2[(size_t)s * E + e] = q;
         }
     }
-    float outv[8];
-    if (do_softmax) {
-        double max_val = sel_v[0];
+    if (t0 >= T) return;  // wave-uniform; no block-wide barrier below
+
+    const int tok = min(t0 + r, T - 1);
+    const bool tok_ok = t0 + r < T;
+    const float* xrow = x + (size_t)tok * H + 8 * g;
+    const uint16_t* wrow[NE];
 #pragma unroll
-        for (int r = 1; r < 8; ++r)
-            if (r < K && sel_v[r] > max_val) max_val = sel_v[r];
+    for (int n = 0; n < NE; ++n) wrow[n] = w + (size_t)min(e_base + 16 * n + r, E - 1) * H + 8 * g;
+
+    f32x4 acc[NE];
+#pragma unroll
+    for (int n = 0; n < NE; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float x2 = 0.f;
+
+    // k-steps of 32; the loads of step i+1 are in flight while step i is converted and multiplied
+    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0;
+    u32x4 b[NE];
+    auto load = [&](int k0) {
+        a0 = *reinterpret_cast<const float4*>(xrow + k0);
+        a1 = *reinterpret_cast<const float4*>(xrow + k0 + 4);
+#pragma unroll
+        for (int n = 0; n < NE; ++n) b[n] = *reinterpret_cast<const u32x4*>(wrow[n] + k0);
+    };
+    if (kbeg < kend) load(kbeg);
+    for (int k0 = kbeg; k0 < kend; k0 += 32) {
+        const float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        u32x4 bb[NE];
+#pragma unroll
+        for (int n = 0; n < NE; ++n) bb[n] = b[n];
+        if (k0 + 32 < kend) load(k0 + 32);
+        u32x4 hi, lo;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t h2 = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+            hi[i] = h2;
+            lo[i] = pack_bf16x2(v[2 * i] - __uint_as_float(h2 << 16), v[2 * i + 1] - __uint_as_float(h2 & 0xFFFF0000u));
+            x2 = fmaf(v[2 * i], v[2 * i], x2);
+            x2 = fmaf(v[2 * i + 1], v[2 * i + 1], x2);
+        }
+        if (first_group && tok_ok && x_bf16) *reinterpret_cast<u32x4*>(x_bf16 + (size_t)tok * H + 8 * g + k0) = hi;
+#pragma unroll
+        for (int n = 0; n < NE; ++n) {
+            acc[n] = mfma_16x16x32(hi, bb[n], acc[n]);
+            acc[n] = mfma_16x16x32(lo, bb[n], acc[n]);
+        }
+    }
+    // accumulator layout: lane holds tokens t0 + 4g + i (i = 0..3) for expert e_base + 16n + r
+#pragma unroll
+    for (int n = 0; n < NE; ++n) {
+        const int e = e_base + 16 * n + r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = t0 + 4 * g + i;
+            if (e < E && t < T) partial[((size_t)s * T + t) * E + e] = acc[n][i];
+        }
+    }
+    if (first_group) {
+        x2 += __shfl_xor(x2, 16, 64);
+        x2 += __shfl_xor(x2, 32, 64);
+        if (g == 0 && tok_ok) xn2[(size_t)s * T + tok] = x2;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Second pass of the two-pass router: one wave per token.
+//   1. approximate scores a[e] = float(sum_s partial[s][t][e]) + bias[e] from the screening pass,
+//      each within d of the exact score, d = err_coeff * |x_t|_2 * max_e |w_e|_2 (Cauchy-Schwarz
+//      on sum|w_k x_k|; err_coeff from the screening pass's error model) plus the final roundings;
+//   2. vK = K-th largest a.  An expert with a[e] < vK - 2d has an exact score below those of the K
+//      experts with a >= vK, so the exact top K lies inside C = {e : a[e] >= vK - 2d};
+//   3. the exact score (fp32 products, fp64 sum: src/run.cpp:341-354, 635-637) of every member
+//      of C, each lane summing its own k in ascending order, lanes combined by a butterfly;
+//   4. top-k and softmax over those exact scores, as in router_finalize_kernel.
+// The result equals router_partial_kernel + router_finalize_kernel up to the order of
+// the fp64 additions; |C| is K except for near-ties at the boundary (every exact tie is in C).
+// grid = ceil(T/4), block = 256, dynamic LDS = 4 * 3 * E * 4 bytes.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void router_refine_kernel(const float* __restrict__ partial, int S,
+                                                            const float* __restrict__ wn2,
+                                                            const float* __restrict__ xn2,
+                                                            const float* __restrict__ x,
+                                                            const uint16_t* __restrict__ w,
+                                                            const uint16_t* __restrict__ bias, float err_coeff,
+                                                            float* __restrict__ topk_v, int* __restrict__ topk_i,
+                                                            int T, int H, int E, int K, int do_softmax) {
+    extern __shared__ float sc[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= T) return;  // no block-wide barrier below
+    float* approx = sc + (size_t)wave * 3 * E;
+    float* exact = approx + E;
+    int* cand = reinterpret_cast<int*>(exact + E);
+
+    float x2 = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < S; ++s) x2 += xn2[(size_t)s * T + t];
+    float w2max = 0.f, amax = 0.f;
+#pragma nounroll
+    for (int e = lane; e < E; e += 64) {
         double sum = 0.0;
+        float q = 0.f;
+#pragma unroll 4
+        for (int s = 0; s < S; ++s) {
+            sum += (double)partial[((size_t)s * T + t) * E + e];
+            q += wn2[(size_t)s * E + e];
+        }
+        const float v = (float)sum + bf16_bits_to_f32(bias[e]);
+        approx[e] = v;
+        exact[e] = -INFINITY;
+        w2max = fmaxf(w2max, q);
+        amax = fmaxf(amax, fabsf(v));
+    }
+    w2max = wave_max_nonneg(w2max);
+    amax = wave_max_nonneg(amax);
+    // upper bound of |approx - exact| for every expert of this token; the 1.001 factors cover the
+    // rounding of the two norms themselves, the last term the final roundings of both scores
+    const float delta = err_coeff * (sqrtf(x2) * 1.001f) * (sqrtf(w2max) * 1.001f) + amax * 0x1p-20f;
+    __builtin_amdgcn_wave_barrier();
+
+    float my_v;
+    int my_i;
+    select_topk(approx, E, K, lane, my_v, my_i);
+    const float thr = lane_value(my_v, K - 1) - 2.f * delta;
+
+    int n_cand = 0;
+#pragma nounroll
+    for (int e0 = 0; e0 < E; e0 += 64) {
+        const int e = e0 + lane;
+        const bool in = e < E && approx[e] >= thr;
+        const unsigned long long ballot = __ballot(in);
+        if (in) cand[n_cand + __popcll(ballot & ((1ull << lane) - 1ull))] = e;
+        n_cand += __popcll(ballot);
+    }
+    if (n_cand < K) {  // not-a-number scores: no screening, every expert is scored exactly
+        for (int e = lane; e < E; e += 64) cand[e] = e;
+        n_cand = E;
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    // exact scores, four candidates at a time (their loads and reductions overlap); lane l takes
+    // float4 number l, l + 64, ... of the token's activations, in ascending order
+    const int n4 = H >> 2;
+    const float4* xrow = reinterpret_cast<const float4*>(x + (size_t)t * H);
+#pragma nounroll
+    for (int c0 = 0; c0 < n_cand; c0 += 4) {
+        const uint2* wrow[4];
+        double acc[4];
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            if (r < K) {
-                outv[r] = expf((float)((double)sel_v[r] - max_val));
-                sum += outv[r];
+        for (int i = 0; i < 4; ++i) {
+            const int e = __builtin_amdgcn_readfirstlane(cand[min(c0 + i, n_cand - 1)]);
+            wrow[i] = reinterpret_cast<const uint2*>(w + (size_t)e * H);
+            acc[i] = 0.0;
+        }
+#pragma unroll 3
+        for (int i4 = lane; i4 < n4; i4 += 64) {
+            const float4 xv = xrow[i4];
+            uint2 wb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) wb[i] = wrow[i][i4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x << 16), xv.x);
+                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x & 0xFFFF0000u), xv.y);
+                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].y << 16), xv.z);
+                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].y & 0xFFFF0000u), xv.w);
             }
         }
 #pragma unroll
-        for (int r = 0; r < 8; ++r)
-            if (r < K) outv[r] = (float)((double)outv[r] / sum);
-    } else {
-#pragma unroll
-        for (int r = 0; r < 8; ++r) outv[r] = sel_v[r];
-    }
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-        if (r < K && lane == r) {
-            topk_v[(size_t)t * K + r] = outv[r];
-            topk_i[(size_t)t * K + r] = sel_i[r];
+        for (int i = 0; i < 4; ++i) {
+            const double total = wave_sum(acc[i]);
+            const int e = __builtin_amdgcn_readfirstlane(cand[min(c0 + i, n_cand - 1)]);
+            if (lane == 0) exact[e] = (float)total + bf16_bits_to_f32(bias[e]);
         }
     }
+    __builtin_amdgcn_wave_barrier();
+
+    select_topk(exact, E, K, lane, my_v, my_i);
+    write_topk(my_v, my_i, K, lane, do_softmax, topk_v + (size_t)t * K, topk_i + (size_t)t * K);
 }
 
 // In-place softmax over the last dimension, one thread per row, the reference's order of
@@ -388,6 +620,59 @@ int launch_router_partial(const float* x, const uint16_t* w, double* partial, ui
         hipLaunchKernelGGL((router_partial_kernel<4, 64>), grid, dim3(256), 0, stream, x, w, partial, x_bf16, T, H, E,
                            seg_len);
     }
+    return launch_status();
+}
+
+// ---- two-pass router -----------------------------------------------------------------------------
+// Worth it once the exact pass is throughput bound (three vector instructions per term); small
+// batches are latency bound and keep the single exact pass.
+bool router_two_pass(int T, int E, int H) { return (long long)T * E >= 65536 && H % 32 == 0; }
+
+static int screen_tiles(int E) { return E <= 16 ? 1 : E <= 32 ? 2 : 4; }  // 16-expert tiles per wave
+
+static int router_screen_segments(int T, int E, int H) {
+    const long long waves_one = (long long)ceil_div(T, 16) * ceil_div(E, 16 * screen_tiles(E));
+    int S = 1;
+    while (S < 16 && waves_one * S < 2048 && H / (S * 2) >= 64) S *= 2;
+    return S;
+}
+
+size_t router_screen_bytes(int T, int E, int H) {
+    const size_t S = router_screen_segments(T, E, H);
+    return S * T * E * sizeof(float) + S * E * sizeof(float) + S * T * sizeof(float);
+}
+
+int launch_router_two_pass(const float* x, const uint16_t* w, const uint16_t* bias, void* scratch, uint16_t* x_bf16,
+                           float* topk_v, int* topk_i, int T, int H, int E, int K, int do_softmax,
+                           hipStream_t stream, hipEvent_t between) {
+    int S = router_screen_segments(T, E, H);
+    const int seg_len = ceil_div(ceil_div(H, S), 32) * 32;
+    S = ceil_div(H, seg_len);  // rounding the segment up can empty the last ones
+    float* partial = static_cast<float*>(scratch);
+    float* wn2 = partial + (size_t)S * T * E;
+    float* xn2 = wn2 + (size_t)S * E;
+    const int ne = screen_tiles(E);
+    dim3 grid(ceil_div(T, 64), ceil_div(E, 16 * ne), S);
+    if (ne == 1) {
+        hipLaunchKernelGGL((router_screen_kernel<1>), grid, dim3(256), 0, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
+                           seg_len);
+    } else if (ne == 2) {
+        hipLaunchKernelGGL((router_screen_kernel<2>), grid, dim3(256), 0, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
+                           seg_len);
+    } else {
+        hipLaunchKernelGGL((router_screen_kernel<4>), grid, dim3(256), 0, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
+                           seg_len);
+    }
+    int rc = launch_status();
+    if (rc) return rc;
+    if (between) MOE_RETURN_IF_HIP(hipEventRecord(between, stream));
+    // error model of the screening pass per unit of |x| |w|: 33 + 2 * k-steps roundings of 2^-23 inside
+    // a segment, the 2^-16 the two bf16 pieces leave out, and 8 * 2^-24 for the product roundings of
+    // the exact path; 1 % slack
+    const float err_coeff = ((float)(33 + 2 * (seg_len / 32)) * 0x1p-23f + 0x1p-16f + 8 * 0x1p-24f) * 1.01f;
+    hipLaunchKernelGGL(router_refine_kernel, dim3(ceil_div(T, 4)), dim3(256),
+                       (size_t)4 * 3 * E * sizeof(float), stream, partial, S, wn2, xn2, x, w, bias, err_coeff, topk_v,
+                       topk_i, T, H, E, K, do_softmax);
     return launch_status();
 }
 

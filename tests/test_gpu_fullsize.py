@@ -50,8 +50,9 @@ def properties(pkg, blk, x, y, ti, tv, shape):
     assert torch.equal(tip, ti[perm]) and torch.equal(tvp, tv[perm])
     assert torch.equal(yp, y[perm])
     # the router's strict summation order selects the same experts
-    ys, tis, _ = blk.forward(x, flags=pkg.MOE_FLAG_ROUTER_STRICT_ORDER)
+    ys, tis, tvs = blk.forward(x, flags=pkg.MOE_FLAG_ROUTER_STRICT_ORDER)
     assert torch.equal(tis, ti)
+    assert torch.allclose(tvs, tv, rtol=1e-6, atol=0)
 
 
 def test_decode256_bf16_and_the_cpu_64_token_case(pkg, wl, oracle, dev):

@@ -231,6 +231,54 @@ def test_block_residual_and_rmsnorm_glue(pkg, wl, oracle, dev):
     assert hostgen.rel_err(xres.cpu().numpy(), x_ref) <= OUT_TOL
 
 
+def test_two_pass_router_near_ties(pkg, oracle, dev):
+    """Large batches take the two-pass router (fp32 screening, exact scores of the candidates).
+    Router rows that are equal, or differ by one bf16 step in a few elements, put many tokens'
+    K-th and (K+1)-th scores closer together than the screening error: indices must still be the
+    oracle's, ties to the lower index, and the weights the exact softmax's."""
+    T, H, I, E, K = 1024, 256, 64, 64, 4
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    x[5] = 0.0                      # every score equals its bias
+    x[6] = x[7]                     # duplicate tokens
+    w = rng.standard_normal((E, H)) * 0.02
+    base = rng.standard_normal(H) * 0.08
+    w_bits = oracle.f32_to_bf16(w)
+    base_bits = oracle.f32_to_bf16(base)
+    for e in (3, 9, 10, 20, 41, 63):  # a family of near-copies that usually wins
+        w_bits[e] = base_bits
+    w_bits[10, 17] += 1             # one bf16 step up in one element
+    w_bits[20, 100] -= 1
+    w_bits[41, 0:4] += 1
+    w_bits[63, 200] += 2
+    b_bits = oracle.f32_to_bf16(rng.standard_normal(E) * 0.01)
+    b_bits[[3, 9, 10, 20, 41, 63]] = b_bits[3]
+    w1 = oracle.f32_to_bf16(rng.standard_normal((E, 2 * I, H)) * 0.05)
+    b1 = oracle.f32_to_bf16(rng.standard_normal((E, 2 * I)) * 0.05)
+    w2 = oracle.f32_to_bf16(rng.standard_normal((E, H, I)) * 0.05)
+    b2 = oracle.f32_to_bf16(rng.standard_normal((E, H)) * 0.05)
+    blk = pkg.MoeBlock(H, I, E, K, *[to_dev(a, dev, True) for a in (w_bits, b_bits, w1, b1, w2, b2)], max_tokens=T)
+    xd = to_dev(x, dev)
+    say("two-pass router, near ties")
+    y, ti, tv = blk.forward(xd)                                            # two-pass
+    scores = torch.empty((T, E), dtype=torch.float32, device=dev)
+    y1, ti1, tv1 = blk.forward(xd, router_score=scores)                    # single exact pass
+    torch.cuda.synchronize()
+    f = oracle.bf16_to_f32
+    ref_y, ref_i, ref_v, ref_s = oracle.moe_block(x, f(w_bits), f(b_bits), f(w1), f(b1), f(w2), f(b2), K, 7.0,
+                                                  want_scores=True)
+    assert np.array_equal(scores.cpu().numpy(), ref_s)
+    top = np.sort(ref_s, axis=1)[:, ::-1]
+    say("  tokens whose K-th and (K+1)-th exact scores are equal: %d, within 1e-4: %d"
+        % (int((top[:, K - 1] == top[:, K]).sum()), int((top[:, K - 1] - top[:, K] < 1e-4).sum())))
+    assert (top[:, K - 1] - top[:, K] < 1e-4).sum() > T // 10  # the case really is exercised
+    assert np.array_equal(ti1.cpu().numpy(), ref_i)
+    assert np.array_equal(ti.cpu().numpy(), ref_i)
+    np.testing.assert_allclose(tv.cpu().numpy(), ref_v, rtol=2e-6)
+    assert torch.equal(ti[6], ti[7]) and torch.equal(y[6], y[7])
+    assert hostgen.rel_err(y.cpu().numpy(), ref_y) <= OUT_TOL
+
+
 # ---- the reference's own data flow: gather -> queue -> mlp1 -> mlp2 scatter -> vecadd -------------
 @pytest.mark.parametrize("fmt", ["bf16", "mxfp4"])
 def test_reference_call_sequence(pkg, wl, oracle, dev, fmt):
