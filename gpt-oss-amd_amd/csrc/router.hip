@@ -228,11 +228,23 @@ __global__ __launch_bounds__(256) void router_partial_small_kernel(const float* 
 // When `partial` is NULL the scores are read from `scores_in` instead.
 // grid = ceil(T/4), block = 256, dynamic LDS = 4*E floats.
 // ---------------------------------------------------------------------------------------------
-MOE_DEVICE bool better(float va, int ia, float vb, int ib) { return va > vb || (va == vb && ia < ib); }
 
 // These kernels run their code once per wave, so their time is instruction fetch as much as
 // anything: loops stay rolled (the round and segment counts are wave-uniform anyway).
 //
+// Sort key of a (score, expert) pair: larger key = better candidate.  High word: the score's bits
+// mapped to an unsigned integer in score order (-0 counts as +0, as in the reference's float
+// comparison); low word: ~index, so equal scores order by the lower index.  Key 0 is "nothing".
+MOE_DEVICE uint64_t rank_key(float v, int e) {
+    const uint32_t u = __float_as_uint(v + 0.f);
+    const uint32_t m = u ^ ((uint32_t)((int32_t)u >> 31) | 0x80000000u);
+    return ((uint64_t)m << 32) | (uint32_t)~e;
+}
+MOE_DEVICE float rank_key_value(uint64_t key) {
+    const uint32_t m = (uint32_t)(key >> 32);
+    return __uint_as_float((m & 0x80000000u) ? m ^ 0x80000000u : ~m);
+}
+
 // K rounds of wave-wide argmax over vals[0..E) ordered by (value desc, index asc).  Lane r < K
 // ends up holding the winner of round r in (my_v, my_i).
 MOE_DEVICE void select_topk(const float* vals, int E, int K, int lane, float& my_v, int& my_i) {
@@ -241,31 +253,26 @@ MOE_DEVICE void select_topk(const float* vals, int E, int K, int lane, float& my
     my_i = 0;
 #pragma nounroll
     for (int r = 0; r < K; ++r) {
-        float bv = -INFINITY;
-        int bi = 0x7FFFFFFF;
+        uint64_t best = 0;
 #pragma nounroll
         for (int c = 0, e = lane; e < E; ++c, e += 64) {
-            const float v = vals[e];
-            if (!(taken & (1u << c)) && (bi == 0x7FFFFFFF || better(v, e, bv, bi))) {
-                bv = v;
-                bi = e;
-            }
+            const uint64_t key = (taken >> c) & 1u ? 0ull : rank_key(vals[e], e);
+            best = key > best ? key : best;
         }
-        // wave-wide winner on the DPP path; a lane without a source keeps (any, 0x7FFFFFFF)
-#define MOE_STEP(C, M)                                                                      \
-    {                                                                                       \
-        const float ov = __uint_as_float(dpp_move<C, M>(0u, __float_as_uint(bv)));          \
-        const int oi = (int)dpp_move<C, M>(0x7FFFFFFFu, (uint32_t)bi);                      \
-        const bool take = oi != 0x7FFFFFFF && (bi == 0x7FFFFFFF || better(ov, oi, bv, bi)); \
-        bv = take ? ov : bv;                                                                \
-        bi = take ? oi : bi;                                                                \
+        // wave-wide maximum on the DPP path (a lane without a source sees key 0)
+#define MOE_STEP(C, M)                                                                          \
+    {                                                                                           \
+        const uint64_t o = ((uint64_t)dpp_move<C, M>(0u, (uint32_t)(best >> 32)) << 32) |       \
+                           dpp_move<C, M>(0u, (uint32_t)best);                                  \
+        best = o > best ? o : best;                                                             \
     }
         MOE_DPP_STEPS(MOE_STEP)
 #undef MOE_STEP
-        bv = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(bv), 63));
-        bi = __builtin_amdgcn_readlane(bi, 63);
+        const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(best >> 32), 63);
+        const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)best, 63);
+        const int bi = (int)~lo;
         if (lane == r) {
-            my_v = bv;
+            my_v = rank_key_value((uint64_t)hi << 32);
             my_i = bi;
         }
         if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
@@ -350,14 +357,20 @@ __global__ __launch_bounds__(256) void router_finalize_kernel(const double* __re
 // The same pass writes the bf16 copy of the activations (the hi pieces) for the expert GEMMs, the
 // squared norm of every token's segment (xn2 [S][T]) and, in the blocks of the first token tile,
 // of every router row's segment (wn2 [S][E]).  partial is [S][T][E] fp32.
-// grid = (ceil(T/64), ceil(E/(16*NE)), S), block = 256; seg_len % 32 == 0, H % 32 == 0.
+// The four waves of a block share the router rows of their segment through LDS.
+// grid = (ceil(T/64), ceil(E/(16*NE)), S), block = 256, dynamic LDS = 16*NE*(seg_len+8)*2 bytes;
+// seg_len % 32 == 0, H % 32 == 0.
 // ---------------------------------------------------------------------------------------------
+constexpr int kScreenDepth = 4;  // k-steps whose activation loads are in flight together
+
 template <int NE>
 __global__ __launch_bounds__(256) void router_screen_kernel(const float* __restrict__ x,
                                                             const uint16_t* __restrict__ w,
                                                             float* __restrict__ partial, float* __restrict__ wn2,
                                                             float* __restrict__ xn2, uint16_t* __restrict__ x_bf16,
                                                             int T, int H, int E, int seg_len) {
+    constexpr int D = kScreenDepth;
+    extern __shared__ __attribute__((aligned(16))) uint16_t wl[];  // [16*NE][seg_len + 8]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, g = lane >> 4;
@@ -365,16 +378,45 @@ __global__ __launch_bounds__(256) void router_screen_kernel(const float* __restr
     const int e_base = blockIdx.y * 16 * NE;
     const int s = blockIdx.z;
     const int kbeg = s * seg_len;
-    const int kend = min(H, kbeg + seg_len);
+    const int kend = min(H, kbeg + seg_len);  // kend - kbeg is a positive multiple of 32
+    const int ldw = seg_len + 8;              // row stride 16 bytes off a multiple of 64: rows r, r+1 land 4 banks apart
     const bool first_group = blockIdx.y == 0;
+
+    // activations first: D k-steps (32 values each) per request group, the next group in flight
+    // while the current one is converted and multiplied
+    const int tok = min(t0 + r, T - 1);
+    const bool tok_ok = t0 + r < T;
+    const float* xrow = x + (size_t)tok * H + 8 * g;
+    float4 xa[D][2];
+    auto load_group = [&](int k0) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int k = min(k0 + 32 * d, kend - 32);
+            xa[d][0] = *reinterpret_cast<const float4*>(xrow + k);
+            xa[d][1] = *reinterpret_cast<const float4*>(xrow + k + 4);
+        }
+    };
+    load_group(kbeg);
+
+    // this block's router rows over the segment -> LDS, shared by the four waves
+    {
+        const int cpr = (kend - kbeg) >> 3;  // 16-byte chunks per row
+        for (int idx = threadIdx.x; idx < 16 * NE * cpr; idx += 256) {
+            const int row = idx / cpr, c = idx - row * cpr;
+            const int e = min(e_base + row, E - 1);
+            *reinterpret_cast<u32x4*>(wl + row * ldw + 8 * c) =
+                *reinterpret_cast<const u32x4*>(w + (size_t)e * H + kbeg + 8 * c);
+        }
+    }
+    __syncthreads();
 
     if (blockIdx.x == 0) {  // block-uniform: squared norms of this block's router rows
         for (int i = wave; i < 16 * NE; i += 4) {
             const int e = e_base + i;
             if (e >= E) break;
             float q = 0.f;
-            for (int k = kbeg + lane; k < kend; k += 64) {
-                const float wf = bf16_bits_to_f32(w[(size_t)e * H + k]);
+            for (int k = lane; k < kend - kbeg; k += 64) {
+                const float wf = bf16_bits_to_f32(wl[i * ldw + k]);
                 q = fmaf(wf, wf, q);
             }
             q = wave_sum(q);
@@ -383,48 +425,45 @@ __global__ __launch_bounds__(256) void router_screen_kernel(const float* __restr
     }
     if (t0 >= T) return;  // wave-uniform; no block-wide barrier below
 
-    const int tok = min(t0 + r, T - 1);
-    const bool tok_ok = t0 + r < T;
-    const float* xrow = x + (size_t)tok * H + 8 * g;
-    const uint16_t* wrow[NE];
-#pragma unroll
-    for (int n = 0; n < NE; ++n) wrow[n] = w + (size_t)min(e_base + 16 * n + r, E - 1) * H + 8 * g;
-
     f32x4 acc[NE];
 #pragma unroll
     for (int n = 0; n < NE; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
     float x2 = 0.f;
+    const int wfrag = r * ldw + 8 * g - kbeg;  // element index of this lane's fragment at k = 0
 
-    // k-steps of 32; the loads of step i+1 are in flight while step i is converted and multiplied
-    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0;
-    u32x4 b[NE];
-    auto load = [&](int k0) {
-        a0 = *reinterpret_cast<const float4*>(xrow + k0);
-        a1 = *reinterpret_cast<const float4*>(xrow + k0 + 4);
+    for (int k0 = kbeg; k0 < kend; k0 += 32 * D) {
+        float4 cur[D][2];
 #pragma unroll
-        for (int n = 0; n < NE; ++n) b[n] = *reinterpret_cast<const u32x4*>(wrow[n] + k0);
-    };
-    if (kbeg < kend) load(kbeg);
-    for (int k0 = kbeg; k0 < kend; k0 += 32) {
-        const float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        u32x4 bb[NE];
-#pragma unroll
-        for (int n = 0; n < NE; ++n) bb[n] = b[n];
-        if (k0 + 32 < kend) load(k0 + 32);
-        u32x4 hi, lo;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t h2 = pack_bf16x2(v[2 * i], v[2 * i + 1]);
-            hi[i] = h2;
-            lo[i] = pack_bf16x2(v[2 * i] - __uint_as_float(h2 << 16), v[2 * i + 1] - __uint_as_float(h2 & 0xFFFF0000u));
-            x2 = fmaf(v[2 * i], v[2 * i], x2);
-            x2 = fmaf(v[2 * i + 1], v[2 * i + 1], x2);
+        for (int d = 0; d < D; ++d) {
+            cur[d][0] = xa[d][0];
+            cur[d][1] = xa[d][1];
         }
-        if (first_group && tok_ok && x_bf16) *reinterpret_cast<u32x4*>(x_bf16 + (size_t)tok * H + 8 * g + k0) = hi;
+        if (k0 + 32 * D < kend) load_group(k0 + 32 * D);
 #pragma unroll
-        for (int n = 0; n < NE; ++n) {
-            acc[n] = mfma_16x16x32(hi, bb[n], acc[n]);
-            acc[n] = mfma_16x16x32(lo, bb[n], acc[n]);
+        for (int d = 0; d < D; ++d) {
+            const int k = k0 + 32 * d;
+            if (k < kend) {  // wave-uniform
+                const float v[8] = {cur[d][0].x, cur[d][0].y, cur[d][0].z, cur[d][0].w,
+                                    cur[d][1].x, cur[d][1].y, cur[d][1].z, cur[d][1].w};
+                u32x4 hi, lo;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t h2 = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+                    hi[i] = h2;
+                    lo[i] = pack_bf16x2(v[2 * i] - __uint_as_float(h2 << 16),
+                                        v[2 * i + 1] - __uint_as_float(h2 & 0xFFFF0000u));
+                    x2 = fmaf(v[2 * i], v[2 * i], x2);
+                    x2 = fmaf(v[2 * i + 1], v[2 * i + 1], x2);
+                }
+                if (first_group && tok_ok && x_bf16)
+                    *reinterpret_cast<u32x4*>(x_bf16 + (size_t)tok * H + 8 * g + k) = hi;
+#pragma unroll
+                for (int n = 0; n < NE; ++n) {
+                    const u32x4 b = *reinterpret_cast<const u32x4*>(wl + (wfrag + 16 * n * ldw + k));
+                    acc[n] = mfma_16x16x32(hi, b, acc[n]);
+                    acc[n] = mfma_16x16x32(lo, b, acc[n]);
+                }
+            }
         }
     }
     // accumulator layout: lane holds tokens t0 + 4g + i (i = 0..3) for expert e_base + 16n + r
@@ -458,7 +497,7 @@ __global__ __launch_bounds__(256) void router_screen_kernel(const float* __restr
 // the fp64 additions; |C| is K except for near-ties at the boundary (every exact tie is in C).
 // grid = ceil(T/4), block = 256, dynamic LDS = 4 * 3 * E * 4 bytes.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void router_refine_kernel(const float* __restrict__ partial, int S,
+__global__ __launch_bounds__(256, 4) void router_refine_kernel(const float* __restrict__ partial, int S,
                                                             const float* __restrict__ wn2,
                                                             const float* __restrict__ xn2,
                                                             const float* __restrict__ x,
@@ -467,34 +506,67 @@ __global__ __launch_bounds__(256) void router_refine_kernel(const float* __restr
                                                             float* __restrict__ topk_v, int* __restrict__ topk_i,
                                                             int T, int H, int E, int K, int do_softmax) {
     extern __shared__ float sc[];
+    __shared__ float w2_of_wave[4];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int t = blockIdx.x * 4 + wave;
-    if (t >= T) return;  // no block-wide barrier below
+    const int t = min(blockIdx.x * 4 + wave, T - 1);  // a surplus wave repeats the last token
     float* approx = sc + (size_t)wave * 3 * E;
     float* exact = approx + E;
     int* cand = reinterpret_cast<int*>(exact + E);
 
+    // largest squared router-row norm: the same for every token, so the block's threads share it
+    float w2max = 0.f;
+#pragma nounroll
+    for (int e = threadIdx.x; e < E; e += 256) {
+        float q = 0.f;
+#pragma nounroll
+        for (int s0 = 0; s0 < S; s0 += 16) {
+            float wq[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) wq[i] = wn2[(size_t)min(s0 + i, S - 1) * E + e];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) q += s0 + i < S ? wq[i] : 0.f;
+        }
+        w2max = fmaxf(w2max, q);
+    }
+    // approximate scores: all loads of up to two experts per lane in flight, summed in segment order
+    float amax = 0.f;
+#pragma nounroll
+    for (int e0 = lane; e0 < E; e0 += 128) {
+#pragma nounroll
+        for (int s0 = 0; s0 < S; s0 += 16) {
+            float part[2][16];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int e = min(e0 + 64 * h, E - 1);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) part[h][i] = partial[((size_t)min(s0 + i, S - 1) * T + t) * E + e];
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int e = e0 + 64 * h;
+                double sum = s0 == 0 ? 0.0 : (double)exact[min(e, E - 1)];  // carries the sum when S > 16
+#pragma unroll
+                for (int i = 0; i < 16; ++i) sum += s0 + i < S ? (double)part[h][i] : 0.0;
+                if (e < E) exact[e] = (float)sum;
+            }
+        }
+    }
     float x2 = 0.f;
 #pragma unroll 4
     for (int s = 0; s < S; ++s) x2 += xn2[(size_t)s * T + t];
-    float w2max = 0.f, amax = 0.f;
+    w2max = wave_max_nonneg(w2max);
+    if (lane == 0) w2_of_wave[wave] = w2max;
+    __syncthreads();
+    if (blockIdx.x * 4 + wave >= T) return;  // no block-wide barrier below
+    w2max = fmaxf(fmaxf(w2_of_wave[0], w2_of_wave[1]), fmaxf(w2_of_wave[2], w2_of_wave[3]));
 #pragma nounroll
     for (int e = lane; e < E; e += 64) {
-        double sum = 0.0;
-        float q = 0.f;
-#pragma unroll 4
-        for (int s = 0; s < S; ++s) {
-            sum += (double)partial[((size_t)s * T + t) * E + e];
-            q += wn2[(size_t)s * E + e];
-        }
-        const float v = (float)sum + bf16_bits_to_f32(bias[e]);
+        const float v = exact[e] + bf16_bits_to_f32(bias[e]);
         approx[e] = v;
         exact[e] = -INFINITY;
-        w2max = fmaxf(w2max, q);
         amax = fmaxf(amax, fabsf(v));
     }
-    w2max = wave_max_nonneg(w2max);
     amax = wave_max_nonneg(amax);
     // upper bound of |approx - exact| for every expert of this token; the 1.001 factors cover the
     // rounding of the two norms themselves, the last term the final roundings of both scores
@@ -522,8 +594,11 @@ __global__ __launch_bounds__(256) void router_refine_kernel(const float* __restr
     __builtin_amdgcn_wave_barrier();
 
     // exact scores, four candidates at a time (their loads and reductions overlap); lane l takes
-    // float4 number l, l + 64, ... of the token's activations, in ascending order
+    // float4 number l, l + 64, ... of the token's activations, in ascending order.  The trip count
+    // is the same for every lane (a lane past the end multiplies zeros), so that the loads of
+    // several iterations can be in flight together.
     const int n4 = H >> 2;
+    const int trips = ceil_div(n4, 64);
     const float4* xrow = reinterpret_cast<const float4*>(x + (size_t)t * H);
 #pragma nounroll
     for (int c0 = 0; c0 < n_cand; c0 += 4) {
@@ -535,14 +610,17 @@ __global__ __launch_bounds__(256) void router_refine_kernel(const float* __restr
             wrow[i] = reinterpret_cast<const uint2*>(w + (size_t)e * H);
             acc[i] = 0.0;
         }
-#pragma unroll 3
-        for (int i4 = lane; i4 < n4; i4 += 64) {
+#pragma unroll 4
+        for (int j = 0; j < trips; ++j) {
+            const bool live = lane + 64 * j < n4;
+            const int i4 = min(lane + 64 * j, n4 - 1);
             const float4 xv = xrow[i4];
             uint2 wb[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) wb[i] = wrow[i][i4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
+                if (!live) wb[i] = make_uint2(0u, 0u);  // zero products leave the sum unchanged
                 acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x << 16), xv.x);
                 acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x & 0xFFFF0000u), xv.y);
                 acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].y << 16), xv.z);
@@ -630,37 +708,44 @@ bool router_two_pass(int T, int E, int H) { return (long long)T * E >= 65536 && 
 
 static int screen_tiles(int E) { return E <= 16 ? 1 : E <= 32 ? 2 : 4; }  // 16-expert tiles per wave
 
-static int router_screen_segments(int T, int E, int H) {
-    const long long waves_one = (long long)ceil_div(T, 16) * ceil_div(E, 16 * screen_tiles(E));
-    int S = 1;
-    while (S < 16 && waves_one * S < 2048 && H / (S * 2) >= 64) S *= 2;
-    return S;
+// Segment length (multiple of 32) and count of the screening pass: enough segments for about 2048
+// waves, and short enough for the block's router rows to fit 64 KB of LDS.
+static void screen_plan(int T, int E, int H, int* seg_len, int* S) {
+    const int ne = screen_tiles(E);
+    const long long waves_one = (long long)ceil_div(T, 16) * ceil_div(E, 16 * ne);
+    int want = 1;
+    while (want < 16 && waves_one * want < 2048 && H / (want * 2) >= 64) want *= 2;
+    const int seg_max = (65536 / (2 * 16 * ne) - 8) / 32 * 32;
+    const int seg = min(seg_max, ceil_div(ceil_div(H, want), 32) * 32);
+    *seg_len = seg;
+    *S = ceil_div(H, seg);
 }
 
 size_t router_screen_bytes(int T, int E, int H) {
-    const size_t S = router_screen_segments(T, E, H);
-    return S * T * E * sizeof(float) + S * E * sizeof(float) + S * T * sizeof(float);
+    int seg_len, S;
+    screen_plan(T, E, H, &seg_len, &S);
+    return ((size_t)S * T * E + (size_t)S * E + (size_t)S * T) * sizeof(float);
 }
 
 int launch_router_two_pass(const float* x, const uint16_t* w, const uint16_t* bias, void* scratch, uint16_t* x_bf16,
                            float* topk_v, int* topk_i, int T, int H, int E, int K, int do_softmax,
                            hipStream_t stream, hipEvent_t between) {
-    int S = router_screen_segments(T, E, H);
-    const int seg_len = ceil_div(ceil_div(H, S), 32) * 32;
-    S = ceil_div(H, seg_len);  // rounding the segment up can empty the last ones
+    int seg_len, S;
+    screen_plan(T, E, H, &seg_len, &S);
     float* partial = static_cast<float*>(scratch);
     float* wn2 = partial + (size_t)S * T * E;
     float* xn2 = wn2 + (size_t)S * E;
     const int ne = screen_tiles(E);
     dim3 grid(ceil_div(T, 64), ceil_div(E, 16 * ne), S);
+    const size_t lds = (size_t)16 * ne * (seg_len + 8) * sizeof(uint16_t);
     if (ne == 1) {
-        hipLaunchKernelGGL((router_screen_kernel<1>), grid, dim3(256), 0, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
+        hipLaunchKernelGGL((router_screen_kernel<1>), grid, dim3(256), lds, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
                            seg_len);
     } else if (ne == 2) {
-        hipLaunchKernelGGL((router_screen_kernel<2>), grid, dim3(256), 0, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
+        hipLaunchKernelGGL((router_screen_kernel<2>), grid, dim3(256), lds, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
                            seg_len);
     } else {
-        hipLaunchKernelGGL((router_screen_kernel<4>), grid, dim3(256), 0, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
+        hipLaunchKernelGGL((router_screen_kernel<4>), grid, dim3(256), lds, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
                            seg_len);
     }
     int rc = launch_status();
