@@ -483,6 +483,44 @@ __global__ __launch_bounds__(256) void router_screen_kernel(const float* __restr
     }
 }
 
+// Exact logits of four experts for one token, by one wave: fp32 products, fp64 sums
+// (src/run.cpp:341-354).  Lane l takes float4 number l, l + 64, ... of the token's activations in
+// ascending order; the lanes' sums are combined by wave_sum's fixed tree.  The trip count is the
+// same for every lane (a lane past the end multiplies zeros), so that the loads of several
+// iterations can be in flight together.  Every lane returns all four totals.
+MOE_DEVICE void exact_dots4(const float* __restrict__ x_row, const uint16_t* __restrict__ w, const int (&e)[4], int H,
+                            int lane, double (&total)[4]) {
+    const int n4 = H >> 2;
+    const int trips = ceil_div(n4, 64);
+    const float4* xrow = reinterpret_cast<const float4*>(x_row);
+    const uint2* wrow[4];
+    double acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        wrow[i] = reinterpret_cast<const uint2*>(w + (size_t)e[i] * H);
+        acc[i] = 0.0;
+    }
+#pragma unroll 4
+    for (int j = 0; j < trips; ++j) {
+        const bool live = lane + 64 * j < n4;
+        const int i4 = min(lane + 64 * j, n4 - 1);
+        const float4 xv = xrow[i4];
+        uint2 wb[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wb[i] = wrow[i][i4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (!live) wb[i] = make_uint2(0u, 0u);  // zero products leave the sum unchanged
+            acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x << 16), xv.x);
+            acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x & 0xFFFF0000u), xv.y);
+            acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].y << 16), xv.z);
+            acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].y & 0xFFFF0000u), xv.w);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) total[i] = wave_sum(acc[i]);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Second pass of the two-pass router: one wave per token.
 //   1. approximate scores a[e] = float(sum_s partial[s][t][e]) + bias[e] from the screening pass,
@@ -593,45 +631,18 @@ __global__ __launch_bounds__(256, 4) void router_refine_kernel(const float* __re
     }
     __builtin_amdgcn_wave_barrier();
 
-    // exact scores, four candidates at a time (their loads and reductions overlap); lane l takes
-    // float4 number l, l + 64, ... of the token's activations, in ascending order.  The trip count
-    // is the same for every lane (a lane past the end multiplies zeros), so that the loads of
-    // several iterations can be in flight together.
-    const int n4 = H >> 2;
-    const int trips = ceil_div(n4, 64);
-    const float4* xrow = reinterpret_cast<const float4*>(x + (size_t)t * H);
+    // exact scores of the candidates, four at a time
+    const float* x_row = x + (size_t)t * H;
 #pragma nounroll
     for (int c0 = 0; c0 < n_cand; c0 += 4) {
-        const uint2* wrow[4];
-        double acc[4];
+        int e[4];
+        double total[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int e = __builtin_amdgcn_readfirstlane(cand[min(c0 + i, n_cand - 1)]);
-            wrow[i] = reinterpret_cast<const uint2*>(w + (size_t)e * H);
-            acc[i] = 0.0;
-        }
-#pragma unroll 4
-        for (int j = 0; j < trips; ++j) {
-            const bool live = lane + 64 * j < n4;
-            const int i4 = min(lane + 64 * j, n4 - 1);
-            const float4 xv = xrow[i4];
-            uint2 wb[4];
+        for (int i = 0; i < 4; ++i) e[i] = __builtin_amdgcn_readfirstlane(cand[min(c0 + i, n_cand - 1)]);
+        exact_dots4(x_row, w, e, H, lane, total);
+        if (lane == 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) wb[i] = wrow[i][i4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (!live) wb[i] = make_uint2(0u, 0u);  // zero products leave the sum unchanged
-                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x << 16), xv.x);
-                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x & 0xFFFF0000u), xv.y);
-                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].y << 16), xv.z);
-                acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].y & 0xFFFF0000u), xv.w);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const double total = wave_sum(acc[i]);
-            const int e = __builtin_amdgcn_readfirstlane(cand[min(c0 + i, n_cand - 1)]);
-            if (lane == 0) exact[e] = (float)total + bf16_bits_to_f32(bias[e]);
+            for (int i = 0; i < 4; ++i) exact[e[i]] = (float)total[i] + bf16_bits_to_f32(bias[e[i]]);
         }
     }
     __builtin_amdgcn_wave_barrier();
