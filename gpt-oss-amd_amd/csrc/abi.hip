@@ -395,13 +395,10 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     g.limit = p->swiglu_limit;
     g.format = fmt;
 
-    // eight waves (256 weight rows) per block when that still yields enough blocks to fill the chip
+    // Decode-sized buckets (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of
+    // 32 rows each.  Blocks run in rounds of one per CU, so the cheaper choice is the one with the
+    // smaller rounds x rows-per-block product; more rows per block also re-read the activations less.
     const int est_tiles = std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
-    // measured on MI355X at decode shapes: bf16 weights stream fastest with uniform waves, MXFP4
-    // weights (four times the work per byte) with producer/consumer waves
-    // MXFP4 (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of 32 rows each.
-    // Blocks run in rounds of one per CU, so the cheaper choice is the one with the smaller
-    // rounds x rows-per-block product; more rows per block also re-read the activations less.
     const int kCUs = 256;  // MI355X
     auto pick_consumers = [&](int rows) {
         const int cost10 = ceil_div(ceil_div(rows / 32, 10) * est_tiles, kCUs) * 10;

@@ -20,10 +20,10 @@
 //                                  stage: one 128-bit load + one scale byte per row tile and stage,
 //                                  dequantised in registers to four A operands)
 //
-// Kernels: expert_stream_ws_kernel (decode-sized buckets, producer and consumer waves, the one the
-// fused block uses), expert_stream_kernel / expert_stream_queue_kernel (uniform waves, activations
-// staged through registers; serve the reference-signature entries), expert_prefill_kernel
-// (128-token blocks, 64 x 128 tile per wave).
+// Kernels: expert_stream_ws_kernel (decode-sized buckets, producer and consumer waves) and
+// expert_prefill_kernel (128-token blocks, 64 x 128 tile per wave) are what the fused block uses;
+// expert_stream_queue_kernel (uniform waves, fp32 activations staged through registers) serves the
+// entries that keep the reference's signatures and work queue.
 #include <type_traits>
 
 #include "common.h"
@@ -685,19 +685,6 @@ MOE_DEVICE void stream_dispatch(const ExpertGemmArgs& a, uint8_t* lds, int e, in
     }
 }
 
-// Token blocks from the bucketing kernel's tile map.  grid = (ceil(row units / WAVES), max_tiles).
-template <int FMT, int R, int EPI, int WAVES>
-__global__ __launch_bounds__(WAVES * 64, 4) void expert_stream_kernel(ExpertGemmArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kLdsStageBytes];
-    const int tile = blockIdx.y;
-    if (tile >= *a.n_tiles) return;  // block-uniform
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * WAVES + wave;
-    const bool active = unit < (a.rows / 64) * (4 / R);
-    stream_dispatch<FMT, R, EPI, false, WAVES>(a, lds, a.tile_expert[tile], a.tile_row0[tile], a.tile_rows[tile],
-                                               unit, active);
-}
-
 // Token blocks from a queue of (expert, row_offset, row_count) triples (entry format of
 // src/hip/scheduler.hip:163-166).  grid = (ceil(row units / 4), token blocks per entry, entries).
 template <int FMT, int R, int EPI>
@@ -878,8 +865,8 @@ MOE_DEVICE void prefill_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int r
     }
 }
 
-// WAVES = 4: two blocks of four waves per CU (their barriers are independent, so one block's
-// stage hand-over overlaps the other's MFMAs); WAVES = 8: one block of eight.
+// Two blocks of WAVES = 4 waves per CU: their barriers are independent, so one block's stage
+// hand-over overlaps the other's MFMAs (one block of eight waves measured slower).
 template <int FMT, int EPI, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, 2) void expert_prefill_kernel(ExpertGemmArgs a) {
     constexpr int NTMAX = 8;
@@ -919,21 +906,14 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
         if (a.waves_per_block == 16) {
             dim3 grid(ceil_div(a.rows / 64, 4), a.max_tiles);
             hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 0, stream, a);
-        } else if (a.waves_per_block == 17) {
-            dim3 grid(ceil_div(a.rows / 64, 8), a.max_tiles);
-            hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 8>), grid, dim3(512), 0, stream, a);
         } else if (a.waves_per_block == 0) {
             dim3 grid(max(a.row_blocks, ceil_div(a.rows / 32, 10)), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, a);
         } else if (a.waves_per_block == 1) {
             dim3 grid(max(a.row_blocks, ceil_div(a.rows / 32, 12)), a.max_tiles);
             hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, a);
-        } else if (a.waves_per_block == 8) {
-            dim3 grid(ceil_div(units, 8), a.max_tiles);
-            hipLaunchKernelGGL((expert_stream_kernel<FMT, R, EPI, 8>), grid, dim3(512), 0, stream, a);
         } else {
-            dim3 grid(ceil_div(units, 4), a.max_tiles);
-            hipLaunchKernelGGL((expert_stream_kernel<FMT, R, EPI, 4>), grid, dim3(256), 0, stream, a);
+            return MOE_ERR_FORMAT;
         }
     } else {
         return MOE_ERR_FORMAT;

@@ -68,9 +68,9 @@ struct ExpertGemmArgs {
     int max_tiles;
     int format;
     int row_blocks;             // producer-consumer kernel: row blocks per token block (0 = as few as fit)
-    int waves_per_block;        // kernel choice: 0 / 1 producer-consumer kernel with 10 / 12 consumer waves (+ 2
-                                // producers); 8 or 4 uniform waves, 64-token blocks; 16 / 17 prefill kernel
-                                // (4 / 8 waves, 128-token blocks)
+    int waves_per_block;        // kernel choice of the fused block: 0 / 1 producer-consumer kernel with 10 / 12
+                                // consumer waves (+ 2 producers), 64-token blocks; 16 prefill kernel (4 waves,
+                                // 128-token blocks).  Ignored by the work-queue entries.
 };
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
 
