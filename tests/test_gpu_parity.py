@@ -279,6 +279,37 @@ def test_two_pass_router_near_ties(pkg, oracle, dev):
     assert hostgen.rel_err(y.cpu().numpy(), ref_y) <= OUT_TOL
 
 
+@pytest.mark.parametrize("T,H,I,E,K", [(300, 320, 64, 250, 4), (20000, 64, 64, 4, 2), (70, 128, 64, 1024, 8),
+                                       (4100, 2880, 64, 17, 4)])
+def test_two_pass_router_odd_shapes(pkg, oracle, dev, T, H, I, E, K):
+    """The two-pass router at shapes that leave partial tiles everywhere: expert counts that are no
+    multiple of 16, token counts that are no multiple of 64, one and many k-segments."""
+    rng = np.random.default_rng(T + E)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    w_bits = oracle.f32_to_bf16(rng.standard_normal((E, H)) * 0.05)
+    b_bits = oracle.f32_to_bf16(rng.standard_normal(E) * 0.05)
+    w1 = oracle.f32_to_bf16(rng.standard_normal((E, 2 * I, H)) * 0.05)
+    b1 = oracle.f32_to_bf16(rng.standard_normal((E, 2 * I)) * 0.05)
+    w2 = oracle.f32_to_bf16(rng.standard_normal((E, H, I)) * 0.05)
+    b2 = oracle.f32_to_bf16(rng.standard_normal((E, H)) * 0.05)
+    blk = pkg.MoeBlock(H, I, E, K, *[to_dev(a, dev, True) for a in (w_bits, b_bits, w1, b1, w2, b2)], max_tokens=T)
+    say("two-pass router", (T, H, I, E, K))
+    y, ti, tv = blk.forward(to_dev(x, dev))
+    torch.cuda.synchronize()
+    f = oracle.bf16_to_f32
+    # router and top-k of the oracle on every token (cheap); the whole block on a few
+    want_s = np.stack([oracle.matmul(x[t], f(w_bits)) + f(b_bits) for t in range(0, T, max(1, T // 512))])
+    sub = np.arange(0, T, max(1, T // 512))
+    want_i = np.argsort(-want_s, axis=1, kind="stable")[:, :K]
+    assert np.array_equal(ti.cpu().numpy()[sub], want_i)
+    few = sub[:24]
+    ref_y, ref_i, ref_v, _ = oracle.moe_block(x[few], f(w_bits), f(b_bits), f(w1), f(b1), f(w2), f(b2), K, 7.0,
+                                              want_scores=True)
+    assert np.array_equal(ti.cpu().numpy()[few], ref_i)
+    np.testing.assert_allclose(tv.cpu().numpy()[few], ref_v, rtol=2e-6)
+    assert hostgen.rel_err(y.cpu().numpy()[few], ref_y) <= OUT_TOL
+
+
 # ---- the reference's own data flow: gather -> queue -> mlp1 -> mlp2 scatter -> vecadd -------------
 @pytest.mark.parametrize("fmt", ["bf16", "mxfp4"])
 def test_reference_call_sequence(pkg, wl, oracle, dev, fmt):
