@@ -19,11 +19,17 @@ inline hipStream_t as_stream(moe_stream_t s) { return reinterpret_cast<hipStream
 constexpr int kStreamTileTokens = 64;
 constexpr int kPrefillTileTokens = 128;
 
-// Prefill kernels once the average bucket fills most of a 128-token block.
-inline bool use_prefill_kernels(int T, int K, int E, unsigned flags) {
+// Which family runs the expert GEMMs, by average bucket size T*K/E (measured crossovers, 20b
+// shapes, token counts 256..4096).  MXFP4: the 128-token-block kernels win as soon as buckets start
+// to overflow one 64-token block (the streaming kernel then reads an expert's weights once per
+// block of its bucket).  bf16: the streaming kernel stays ahead up to a few hundred rows per expert
+// (the second block of a bucket finds the weights in the Infinity Cache, and the 128-token bf16
+// kernel has no direct-to-LDS staging).
+inline bool use_prefill_kernels(int T, int K, int E, int format, unsigned flags) {
     if (flags & MOE_FLAG_FORCE_STREAM) return false;
     if (flags & MOE_FLAG_FORCE_TILED) return true;
-    return (long long)T * K >= 96LL * E;
+    const long long rows = (long long)T * K;
+    return format == MOE_WEIGHTS_MXFP4_TILED ? rows >= 52LL * E : rows >= 448LL * E;
 }
 
 // Carves the caller's workspace for moe_block_forward; with base == nullptr only sizes it.
@@ -374,7 +380,7 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     if ((rc = mark())) return rc;
 
     // 2. bucketing + token-block map  (src/forward.cpp:329-376)
-    const bool prefill = use_prefill_kernels(T, K, E, p->flags);
+    const bool prefill = use_prefill_kernels(T, K, E, p->weight_format, p->flags);
     const int tile_tokens = prefill ? kPrefillTileTokens : kStreamTileTokens;
     const int max_tiles = tile_map_capacity(T * K, E, tile_tokens);  // <= ws.max_tiles (sized for 64)
     TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles};

@@ -177,7 +177,7 @@ SMALL = [
     (17, 2880, 2880, 4, 2, "mxfp4"),     # real row/contraction lengths, few experts
     (64, 512, 256, 8, 4, "mxfp4"),       # contraction lengths that are whole groups of four stages / two stages
     (64, 512, 256, 8, 4, "bf16"),
-    # prefill-sized buckets (T*K >= 96*E): 128-token blocks, every token-tile count from 1 to 8
+    # large buckets: every token-tile count from 1 to 8 in the 128-token-block kernels
     (300, 128, 64, 4, 4, "bf16"),
     (700, 320, 192, 8, 4, "mxfp4"),      # ragged last MX chunk on the gate/up side
     (700, 320, 192, 8, 4, "bf16"),
@@ -209,6 +209,12 @@ def test_block_small(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
     # strict router order gives the same routing, and the whole call is deterministic
     y2, ti2, tv2 = blk.forward(x, flags=pkg.MOE_FLAG_ROUTER_STRICT_ORDER)
     assert torch.equal(ti2, ti) and torch.equal(y2, y) and torch.equal(tv2, tv)
+    # both kernel families on every shape, whichever the size rule picked above
+    for name, flag in (("64-token blocks", pkg.MOE_FLAG_FORCE_STREAM), ("128-token blocks", pkg.MOE_FLAG_FORCE_TILED)):
+        yf, tif, _ = blk.forward(x, flags=flag)
+        errf = hostgen.rel_err(yf.cpu().numpy(), ref_y)
+        say("  %s: rel err %.3e" % (name, errf))
+        assert torch.equal(tif, ti) and errf <= OUT_TOL
 
 
 def test_block_residual_and_rmsnorm_glue(pkg, wl, oracle, dev):
