@@ -217,6 +217,39 @@ def test_block_small(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
         assert torch.equal(tif, ti) and errf <= OUT_TOL
 
 
+def _random_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        E = int(rng.choice([2, 3, 5, 8, 13, 32, 40]))
+        K = int(rng.integers(1, min(8, E) + 1))
+        T = int(rng.choice([1, 2, 7, 31, 64, 65, 129, 257, 400]))
+        H = 64 * int(rng.integers(1, 9))
+        I = 64 * int(rng.integers(1, 5))
+        out.append((T, H, I, E, K, "bf16" if i % 2 else "mxfp4"))
+    return out
+
+
+@pytest.mark.parametrize("T,H,I,E,K,fmt", _random_shapes(24, seed=20))
+def test_block_random_shapes(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
+    """Seeded random small shapes (one and many tokens, K from 1 to 8, expert counts that are no power
+    of two), each through the size rule's choice and through both forced kernel families."""
+    shape = wl.MoeShape("rand", T=T, H=H, I=I, E=E, K=K, fmt=fmt, seed=1000 + T + 7 * H + E)
+    say("block_random", shape)
+    table = oracle.normal_table()
+    blk, raw = wl.make_device_layer(shape, table, dev)
+    x = wl.make_device_input(shape, table, dev)
+    hw = hostgen.host_layer(oracle, wl, shape)
+    ref_y, ref_i, ref_v, _ = hostgen.oracle_block(oracle, shape, hw, hostgen.host_input(oracle, wl, shape))
+    for flags in (0, pkg.MOE_FLAG_FORCE_STREAM, pkg.MOE_FLAG_FORCE_TILED):
+        y, ti, tv = blk.forward(x, flags=flags)
+        torch.cuda.synchronize()
+        assert np.array_equal(ti.cpu().numpy(), ref_i), flags
+        np.testing.assert_allclose(tv.cpu().numpy(), ref_v, rtol=2e-6)
+        err = hostgen.rel_err(y.cpu().numpy(), ref_y)
+        assert err <= OUT_TOL, (flags, err)
+
+
 def test_block_residual_and_rmsnorm_glue(pkg, wl, oracle, dev):
     shape = wl.MoeShape("glue", T=40, H=256, I=128, E=8, K=4, fmt="bf16", seed=3)
     table = oracle.normal_table()
