@@ -98,6 +98,23 @@ def test_prefill4096_mxfp4_zipf(pkg, wl, oracle, dev):
     assert hostgen.rel_err(ys.cpu().numpy(), y.cpu().numpy()) <= 1e-5
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "mxfp4"])
+def test_largest_batch(pkg, wl, oracle, dev, fmt):
+    """The documented maximum of 65535 tokens per call (small H and I keep it cheap): every launch grid
+    and the workspace carving at their limits; a spread of tokens against the oracle, the rest
+    through the size-independent properties."""
+    shape = wl.MoeShape("maxT", T=65535, H=64, I=64, E=16, K=2, fmt=fmt, seed=9)
+    say("largest batch", shape)
+    blk, raw, x, y, ti, tv = run_block(wl, oracle, dev, shape)
+    tokens = np.unique(np.concatenate([np.arange(8), np.arange(65527, 65535),
+                                       np.random.default_rng(1).integers(0, 65535, 48)]))
+    check_tokens(wl, oracle, shape, x, y, ti, tv, tokens)
+    counts = np.bincount(ti.cpu().numpy().ravel(), minlength=shape.E)
+    assert counts.sum() == 65535 * 2
+    properties(pkg, blk, x, y, ti, tv, shape)
+    assert pkg.block_workspace_bytes(65536, 64, 64, 16, 2) == 0  # one more token is refused
+
+
 def test_stack120b_mxfp4(pkg, wl, oracle, dev):
     """Config 5: 36 layers, 128 experts, 1024 tokens, all weights (~61 GB) resident on one GPU.
     Layer glue as the reference's: t = rmsnorm(x) (unit weight), x += moe(t)."""
