@@ -62,6 +62,8 @@ class BlockParams(_c.Structure):
         ("workspace", _vp),
         ("workspace_bytes", _sz),
         ("flags", _c.c_uint32),
+        ("next_norm_weight", _vp),
+        ("next_norm_out", _vp),
     ]
 
 
@@ -301,7 +303,8 @@ class MoeBlock:
             raise MoeError("moe_block_workspace_bytes", -4)
         self.workspace = workspace  # layers run one after another on a stream may share it
 
-    def params(self, t, e_agg, topk_i, topk_v, router_score=None, residual_x=None, flags=0):
+    def params(self, t, e_agg, topk_i, topk_v, router_score=None, residual_x=None, flags=0, next_norm_weight=None,
+               next_norm_out=None):
         T = t.shape[0]
         p = BlockParams()
         p.struct_bytes = ctypes.sizeof(BlockParams)
@@ -315,10 +318,11 @@ class MoeBlock:
         p.router_score, p.residual_x = _ptr(router_score), _ptr(residual_x)
         p.workspace, p.workspace_bytes = _ptr(self.workspace), self.workspace.numel()
         p.flags = flags
+        p.next_norm_weight, p.next_norm_out = _ptr(next_norm_weight), _ptr(next_norm_out)
         return p
 
     def forward(self, t, e_agg=None, topk_i=None, topk_v=None, router_score=None, residual_x=None, flags=0,
-                stream=None):
+                stream=None, next_norm_weight=None, next_norm_out=None):
         T = t.shape[0]
         dev = t.device
         if e_agg is None:
@@ -327,7 +331,7 @@ class MoeBlock:
             topk_i = torch.empty((T, self.K), dtype=torch.int32, device=dev)
         if topk_v is None:
             topk_v = torch.empty((T, self.K), dtype=torch.float32, device=dev)
-        p = self.params(t, e_agg, topk_i, topk_v, router_score, residual_x, flags)
+        p = self.params(t, e_agg, topk_i, topk_v, router_score, residual_x, flags, next_norm_weight, next_norm_out)
         _check("moe_block_forward", _lib.moe_block_forward(ctypes.byref(p), _stream(stream)))
         return e_agg, topk_i, topk_v
 

@@ -5,6 +5,8 @@
 #include "kernels.h"
 
 #include <algorithm>
+#include <cstddef>
+#include <cstring>
 #include <new>
 
 using namespace moe;
@@ -270,7 +272,8 @@ int moe_vecadd_and_zero(float* a, float* b, float weight, int batch, int size, m
 
 int moe_rmsnorm(float* o, const float* x, const moe_bf16_t* weight, int batch, int size, moe_stream_t stream) {
     if (!o || !x || !weight) return MOE_ERR_NULL;
-    if (batch <= 0 || size <= 0) return MOE_ERR_SHAPE;
+    if (batch <= 0 || size <= 0 || size % 4 != 0) return MOE_ERR_SHAPE;
+    if ((((uintptr_t)o | (uintptr_t)x) & 15u) || ((uintptr_t)weight & 7u)) return MOE_ERR_ALIGN;
     return launch_rmsnorm(o, x, weight, batch, size, as_stream(stream));
 }
 
@@ -333,9 +336,17 @@ struct moe_stage_timer {
     hipEvent_t ev[MOE_N_STAGES + 1];
 };
 
-static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, moe_stage_timer* timer) {
-    if (!p) return MOE_ERR_NULL;
-    if (p->struct_bytes != sizeof(moe_block_params)) return MOE_ERR_FORMAT;
+static int block_forward_impl(const moe_block_params* caller, moe_stream_t stream_, moe_stage_timer* timer) {
+    if (!caller) return MOE_ERR_NULL;
+    // the struct as it was before next_norm_weight / next_norm_out were appended is still accepted
+    constexpr size_t kOldBytes = offsetof(moe_block_params, next_norm_weight);
+    if (caller->struct_bytes != sizeof(moe_block_params) && caller->struct_bytes != kOldBytes) return MOE_ERR_FORMAT;
+    moe_block_params local{};
+    memcpy(&local, caller, caller->struct_bytes);
+    const moe_block_params* p = &local;
+    if ((p->next_norm_weight != nullptr) != (p->next_norm_out != nullptr)) return MOE_ERR_NULL;
+    if (p->next_norm_out && !p->residual_x) return MOE_ERR_NULL;
+    if (((uintptr_t)p->next_norm_out & 15u) || ((uintptr_t)p->next_norm_weight & 7u)) return MOE_ERR_ALIGN;
     const int T = p->n_tokens, H = p->hidden_dim, I = p->intermediate_dim, E = p->n_experts,
               K = p->experts_per_token;
     int rc = check_dims(T, H, I, E, K);
@@ -470,8 +481,17 @@ static int block_forward_impl(const moe_block_params* p, moe_stream_t stream_, m
     if ((rc = mark())) return rc;
 
     // 5. weighted combine in ascending expert id (+ residual)  (src/run.cpp:702-712)
+    if (p->next_norm_out) {
+        rc = launch_combine_norm(ws.y_by_slot, ws.slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x,
+                                 p->next_norm_weight, p->next_norm_out, T, K, H, stream);
+        if (rc != MOE_ERR_LIMIT) return rc ? rc : mark();
+    }
     rc = launch_combine(ws.y_by_slot, ws.slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x, T, K, H, stream);
     if (rc) return rc;
+    if (p->next_norm_out) {  // rows too long for the fused kernel
+        rc = launch_rmsnorm(p->next_norm_out, p->residual_x, p->next_norm_weight, T, H, stream);
+        if (rc) return rc;
+    }
     return mark();
 }
 

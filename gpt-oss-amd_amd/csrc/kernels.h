@@ -77,6 +77,10 @@ int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
 // ---- combine.hip -------------------------------------------------------------------------------
 int launch_combine(const float* y_by_slot, const int* slot_of, const int* topk_i, const float* topk_v,
                    float* e_agg, float* residual_x, int T, int K, int H, hipStream_t stream);
+// combine + residual add + the RMSNorm that follows; MOE_ERR_LIMIT if H is too long for one pass
+int launch_combine_norm(const float* y_by_slot, const int* slot_of, const int* topk_i, const float* topk_v,
+                        float* e_agg, float* residual_x, const uint16_t* norm_weight, float* norm_out, int T, int K,
+                        int H, hipStream_t stream);
 int launch_vecadd_and_zero(float* a, float* b, float weight, int batch, int size, hipStream_t stream);
 int launch_rmsnorm(float* o, const float* x, const uint16_t* weight, int batch, int size, hipStream_t stream);
 

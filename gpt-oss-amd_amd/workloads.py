@@ -185,7 +185,11 @@ class DeviceStack:
 
     def prepare(self, x):
         """Parameter blocks for forward(x): built once so the timed loop does no Python tensor work."""
-        self.params = [blk.params(self.t, self.e_agg, self.topk_i[l], self.topk_v[l], residual_x=x)
+        # every block but the last also produces the next layer's normalised input (fused into its combine)
+        last = len(self.blocks) - 1
+        self.params = [blk.params(self.t, self.e_agg, self.topk_i[l], self.topk_v[l], residual_x=x,
+                                  next_norm_weight=None if l == last else self.rms_w,
+                                  next_norm_out=None if l == last else self.t)
                        for l, blk in enumerate(self.blocks)]
         self.x = x
 
@@ -194,8 +198,8 @@ class DeviceStack:
         s = torch.cuda.current_stream().cuda_stream if stream is None else stream
         T, H = self.shape.T, self.shape.H
         stop = len(self.blocks) if stop is None else stop
+        _pkg.rmsnorm(self.t, self.x, self.rms_w, T, H, stream=s)  # later layers get theirs from the block before
         for l in range(start, stop):
-            _pkg.rmsnorm(self.t, self.x, self.rms_w, T, H, stream=s)
             self.blocks[l].launch(self.params[l], s)
 
 

@@ -162,7 +162,8 @@ MOE_API int moe_vecadd_and_zero(float* a, float* b, float weight, int batch, int
 
 /* FFN RMSNorm feeding the block (src/hip/rmsnorm.hip:3-45; call site src/forward.cpp:315;
  * arithmetic of src/run.cpp:306-319: fp64 sum of fp32 squares, eps 1e-5f). weight is bf16 as
- * the reference holds it on the device (include/model.hpp:93). */
+ * the reference holds it on the device (include/model.hpp:93).  size % 4 == 0; o and x
+ * 16-byte aligned, weight 8-byte aligned. */
 MOE_API int moe_rmsnorm(float* o, const float* x, const moe_bf16_t* weight, int batch, int size,
                 moe_stream_t stream);
 
@@ -199,7 +200,7 @@ MOE_API int moe_mxfp4_tiled_to_bf16(const uint8_t* tiled_blocks, const uint8_t* 
  * src/run.cpp:628-707 on the CPU, whose arithmetic order it follows).
  * ---------------------------------------------------------------------------------------- */
 typedef struct moe_block_params {
-    uint32_t struct_bytes;   /* sizeof(moe_block_params), for forward compatibility */
+    uint32_t struct_bytes;   /* sizeof(moe_block_params) of the caller's header */
     int32_t n_tokens;        /* B <= 65535 */
     int32_t hidden_dim;      /* H, % 64 == 0 */
     int32_t intermediate_dim;/* I, % 64 == 0 */
@@ -225,6 +226,14 @@ typedef struct moe_block_params {
     void* workspace;         /* moe_block_workspace_bytes(), 256-byte aligned */
     size_t workspace_bytes;
     uint32_t flags;          /* MOE_FLAG_* */
+    /* Optional, both or neither; needs residual_x.  The RMSNorm that follows the residual add in
+     * the layer loop (attention norm of the next layer, src/forward.cpp:262, or the final norm,
+     * :997), done in the combine's pass over the row:
+     *   next_norm_out = rmsnorm(residual_x after the add, next_norm_weight)   (as moe_rmsnorm)
+     * A caller built against the struct without these two members (struct_bytes says so) gets
+     * the behaviour of NULL. */
+    const moe_bf16_t* next_norm_weight; /* [H] */
+    float* next_norm_out;               /* [B,H] */
 } moe_block_params;
 
 enum {

@@ -217,6 +217,43 @@ def test_block_small(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
         assert torch.equal(tif, ti) and errf <= OUT_TOL
 
 
+@pytest.mark.parametrize("T,H", [(40, 256), (130, 2880), (9, 4160)])
+def test_next_norm_fused_into_combine(pkg, wl, oracle, dev, T, H):
+    """residual add + the RMSNorm that follows, done by the block's last kernel: bit-identical to
+    the block without it followed by moe_rmsnorm (rows longer than 4096 take that route inside)."""
+    import ctypes
+    shape = wl.MoeShape("nextnorm", T=T, H=H, I=64, E=8, K=4, fmt="bf16", seed=T)
+    table = oracle.normal_table()
+    blk, raw = wl.make_device_layer(shape, table, dev)
+    t_in = wl.make_device_input(shape, table, dev)
+    x0 = torch.randn((T, H), device=dev, generator=torch.Generator(device=dev).manual_seed(3)) * 2.0
+    w_bits = oracle.f32_to_bf16(1 + 0.2 * np.random.default_rng(1).standard_normal(H))
+    w_d = to_dev(w_bits, dev, True)
+    # separate: block with residual, then the norm
+    xa = x0.clone()
+    ya, tia, tva = blk.forward(t_in, residual_x=xa)
+    na = torch.empty_like(xa)
+    pkg.rmsnorm(na, xa, w_d, T, H)
+    # fused
+    xb = x0.clone()
+    nb = torch.full_like(xb, float("nan"))
+    yb, tib, tvb = blk.forward(t_in, residual_x=xb, next_norm_weight=w_d, next_norm_out=nb)
+    torch.cuda.synchronize()
+    assert torch.equal(ya, yb) and torch.equal(xa, xb) and torch.equal(tia, tib)
+    assert torch.equal(na, nb)
+    ref = np.stack([oracle.rmsnorm(r, oracle.bf16_to_f32(w_bits)) for r in xa.cpu().numpy()])
+    np.testing.assert_allclose(nb.cpu().numpy(), ref, rtol=3e-7, atol=1e-9)
+    # a caller compiled against the struct without the two members still works
+    p = blk.params(t_in, torch.empty_like(ya), tia, tva, residual_x=x0.clone())
+    p.struct_bytes = pkg.BlockParams.next_norm_weight.offset
+    assert pkg.lib.moe_block_forward(ctypes.byref(p), torch.cuda.current_stream().cuda_stream) == 0
+    # both members or neither, and the norm needs the residual
+    p = blk.params(t_in, torch.empty_like(ya), tia, tva, residual_x=x0.clone(), next_norm_weight=w_d)
+    assert pkg.lib.moe_block_forward(ctypes.byref(p), None) == -1
+    p = blk.params(t_in, torch.empty_like(ya), tia, tva, next_norm_weight=w_d, next_norm_out=nb)
+    assert pkg.lib.moe_block_forward(ctypes.byref(p), None) == -1
+
+
 def _random_shapes(n, seed):
     rng = np.random.default_rng(seed)
     out = []
