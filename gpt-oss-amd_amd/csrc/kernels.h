@@ -67,7 +67,8 @@ struct ExpertGemmArgs {
     float alpha, limit;
     int max_tiles;
     int format;
-    int row_blocks;             // producer-consumer kernel: row blocks per token block (0 = as few as fit)
+    int row_blocks;             // row blocks per token block (producer-consumer kernel: 0 = as few as fit;
+                                // prefill kernel: set by the launcher)
     int waves_per_block;        // kernel choice of the fused block: 0 / 1 producer-consumer kernel with 10 / 12
                                 // consumer waves (+ 2 producers), 64-token blocks; 16 prefill kernel (4 waves,
                                 // 128-token blocks).  Ignored by the work-queue entries.
