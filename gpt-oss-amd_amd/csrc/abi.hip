@@ -468,6 +468,9 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     a2.bias_expert_stride = H;
     a2.waves_per_block = pick_kernel(H);
     a2.row_blocks = prefill ? 0 : pick_row_blocks(H, a2.waves_per_block);
+    // measured: the down GEMM gains 4-10 % from keeping a token block on one XCD (its input rows were
+    // written by the gate/up launch just before), the gate/up GEMM loses up to 2 %
+    a2.xcd_tiles = 1;
     if (fmt == MOE_WEIGHTS_BF16) {
         a2.w_expert_stride = (long long)H * I;
     } else {

@@ -638,12 +638,17 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0, bias_raw);
 }
 
-// grid = (ceil(row units / CONS), max_tiles), block = 64 (CONS + PROD); one block per CU: twelve
+// grid = row blocks x token blocks (padded to a multiple of 8), block = 64 (CONS + PROD); one block per CU: twelve
 // waves leave 168 registers per lane, fourteen leave 128.
 template <int FMT, int EPI, int CONS, int PROD>
 __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) void expert_stream_ws_kernel(ExpertGemmArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kWsRing * kLdsStageBytes];
-    const int tile = blockIdx.y;
+    // Linear block index -> (token block, row block).  Workgroups go to the eight XCDs round-robin by
+    // linear index; with a.xcd_tiles all row blocks of a token block run on one XCD (its activations
+    // enter one L2 once), otherwise they are spread over all of them.
+    const int n_rb = a.row_blocks;
+    const int tile = a.xcd_tiles ? ((blockIdx.x >> 3) / n_rb) * 8 + (blockIdx.x & 7) : blockIdx.x / n_rb;
+    const int rb = a.xcd_tiles ? (blockIdx.x >> 3) % n_rb : blockIdx.x % n_rb;
     if (tile >= *a.n_tiles) return;  // block-uniform
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int e = a.tile_expert[tile];
@@ -659,8 +664,8 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
     } else {
         // the row units of the weight matrix are spread evenly over the gridDim.x row blocks
         const int units = a.rows / 32;
-        const int u0 = (int)((long long)blockIdx.x * units / gridDim.x);
-        const int u1 = (int)((long long)(blockIdx.x + 1) * units / gridDim.x);
+        const int u0 = (int)((long long)rb * units / n_rb);
+        const int u1 = (int)((long long)(rb + 1) * units / n_rb);
         const int unit = u0 + wave;
         const bool active = unit < u1;
         if (nt == 4) ws_consumer<FMT, 4, EPI>(a, lds, e, row0, nrows, unit, active);
@@ -917,11 +922,15 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             dim3 grid(ceil_div(a.max_tiles, 8) * 8 * b.row_blocks);  // every XCD gets whole token blocks
             hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 0, stream, b);
         } else if (a.waves_per_block == 0) {
-            dim3 grid(max(a.row_blocks, ceil_div(a.rows / 32, 10)), a.max_tiles);
-            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, a);
+            ExpertGemmArgs b = a;
+            b.row_blocks = max(a.row_blocks, ceil_div(a.rows / 32, 10));
+            dim3 grid(ceil_div(a.max_tiles, 8) * 8 * b.row_blocks);
+            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, b);
         } else if (a.waves_per_block == 1) {
-            dim3 grid(max(a.row_blocks, ceil_div(a.rows / 32, 12)), a.max_tiles);
-            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, a);
+            ExpertGemmArgs b = a;
+            b.row_blocks = max(a.row_blocks, ceil_div(a.rows / 32, 12));
+            dim3 grid(ceil_div(a.max_tiles, 8) * 8 * b.row_blocks);
+            hipLaunchKernelGGL((expert_stream_ws_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, b);
         } else {
             return MOE_ERR_FORMAT;
         }

@@ -69,6 +69,7 @@ struct ExpertGemmArgs {
     int format;
     int row_blocks;             // row blocks per token block (producer-consumer kernel: 0 = as few as fit;
                                 // prefill kernel: set by the launcher)
+    int xcd_tiles;              // producer-consumer kernel: all row blocks of a token block on one XCD
     int waves_per_block;        // kernel choice of the fused block: 0 / 1 producer-consumer kernel with 10 / 12
                                 // consumer waves (+ 2 producers), 64-token blocks; 16 prefill kernel (4 waves,
                                 // 128-token blocks).  Ignored by the work-queue entries.
