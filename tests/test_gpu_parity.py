@@ -137,7 +137,8 @@ def test_topk_ties_go_to_lower_index(pkg, oracle, dev):
 
 
 # ---- bucketing -----------------------------------------------------------------------------------
-@pytest.mark.parametrize("T,K,E", [(1, 1, 1), (7, 2, 4), (256, 4, 32), (4096, 4, 32), (1024, 4, 128), (1500, 8, 1000)])
+@pytest.mark.parametrize("T,K,E", [(1, 1, 1), (7, 2, 4), (256, 4, 32), (4096, 4, 32), (1024, 4, 128), (1500, 8, 1000),
+                                   (1025, 4, 8), (5000, 4, 32), (65535, 2, 16)])
 def test_bucketing_bit_exact(pkg, oracle, dev, T, K, E):
     rng = np.random.default_rng(T + E)
     p = 1.0 / np.arange(1, E + 1) ** 1.2
