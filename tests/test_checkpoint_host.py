@@ -174,3 +174,32 @@ def test_safetensors_dense(ck, tmp_path):
         data, dtype = c.layer_tensor(2, ck.T_W_MLP2)
         assert dtype == ck.DTYPE_BF16
         assert np.array_equal(data, ckptgen.f32_to_bf16_bits(tensors["block.2.mlp.mlp2_weight"]).ravel())
+
+
+def test_upload_rejects_bad_arguments_without_a_device(pkg, ck, tmp_path):
+    """Every argument check of moe_ckpt_upload_layer comes before the first device call."""
+    cfg = ckptgen.TINY
+    path = tmp_path / "m.bin"
+    ckptgen.write_bin(path, cfg, ckptgen.make_tensors(cfg, seed=8, mxfp4=False))
+    with ck.Checkpoint.open_bin(path) as c:
+        up = pkg.lib.moe_ckpt_upload_layer
+        d = ck.LayerDevice()
+        d.struct_bytes = ctypes.sizeof(ck.LayerDevice)
+        need = c.staging_bytes()
+        assert need == 2 * 32 * 64 * 4 and need % 256 == 0
+        fake = 1 << 20  # never dereferenced: each call below fails a check first
+        assert up(c._h, 0, ctypes.byref(d), None, need, None) == -1
+        assert up(None, 0, ctypes.byref(d), fake, need, None) == -1
+        assert up(c._h, 3, ctypes.byref(d), fake, need, None) == -2          # layer out of range
+        assert up(c._h, 0, ctypes.byref(d), fake + 16, need, None) == -6     # staging not 256-byte aligned
+        assert up(c._h, 0, ctypes.byref(d), fake, need - 1, None) == -4      # staging too small
+        d.weight_format = 1
+        assert up(c._h, 0, ctypes.byref(d), fake, need, None) == -5          # tiled MXFP4 from a dense file
+        d.weight_format = 7
+        assert up(c._h, 0, ctypes.byref(d), fake, need, None) == -5
+        d.struct_bytes = 12
+        assert up(c._h, 0, ctypes.byref(d), fake, need, None) == -5
+        # a layer descriptor with every destination NULL uploads nothing and succeeds
+        d = ck.LayerDevice()
+        d.struct_bytes = ctypes.sizeof(ck.LayerDevice)
+        assert up(c._h, 0, ctypes.byref(d), fake, need, None) == 0
