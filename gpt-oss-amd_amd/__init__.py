@@ -73,6 +73,8 @@ SIGNATURES = {
     "moe_error_string": (_c.c_char_p, [_i]),
     "moe_router_scratch_bytes": (_sz, [_i, _i]),
     "moe_gemm_router": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
+    "moe_gemm_router_static_max_bytes": (_sz, []),
+    "moe_gemm_router_static": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "moe_topk": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "moe_softmax": (_i, [_vp, _i, _i, _vp]),
     "moe_bucket_by_expert": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
@@ -149,6 +151,13 @@ def gemm_router(xout, x_batch, w, bias, N, K, M, stream=None, scratch=None):
         scratch = torch.empty(_lib.moe_router_scratch_bytes(N, M), dtype=torch.uint8, device=xout.device)
     _check("moe_gemm_router", _lib.moe_gemm_router(_ptr(xout), _ptr(x_batch), _ptr(w), _ptr(bias), N, K, M,
                                                    _ptr(scratch), scratch.numel(), _stream(stream)))
+
+
+def gemm_router_static(xout, x_batch, w, bias, N, K, M, stream=None):
+    """gemm_router with the reference's exact argument list; scratch is a fixed array inside the library,
+    nothing is allocated (N * M limited: moe_gemm_router_static in include/moe_abi.h)."""
+    _check("moe_gemm_router_static", _lib.moe_gemm_router_static(_ptr(xout), _ptr(x_batch), _ptr(w), _ptr(bias), N, K,
+                                                                 M, _stream(stream)))
 
 
 def topk(topk_values, topk_indices, router_scores, batch_size, num_experts, experts_per_token, stream=None):

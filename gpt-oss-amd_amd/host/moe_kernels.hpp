@@ -7,7 +7,8 @@
 //   * errors come back as return codes (0 = ok) instead of exit(1) inside CHECK_HIP
 //     (include/model.hpp:8-17);
 //   * gemm_router needs a scratch buffer (fp64 partial sums): pass one through
-//     moe_router_scratch(), sized by moe_router_scratch_bytes();
+//     moe_router_scratch(), sized by moe_router_scratch_bytes(); without one the call goes to
+//     moe_gemm_router_static (fixed 16 MiB array inside the library, N * M limited);
 //   * bucketing is one call (bucket_by_expert) instead of memset + three kernels
 //     (src/forward.cpp:333-349), and there is one work queue instead of a heavy and a light one;
 //   * __hip_bfloat16 pointers are passed as moe_bf16_t* (same size and bit layout).
@@ -31,6 +32,8 @@ inline RouterScratch& moe_router_scratch() {
 inline int gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias, int N, int K,
                        int M, moe_stream_t stream = nullptr) {
     RouterScratch& s = moe_router_scratch();
+    // no registered buffer: the variant whose scratch is a fixed array inside the library
+    if (!s.ptr) return moe_gemm_router_static(xout, x_batch, w, bias, N, K, M, stream);
     return moe_gemm_router(xout, x_batch, w, bias, N, K, M, s.ptr, s.bytes, stream);
 }
 

@@ -76,6 +76,21 @@ MOE_API size_t moe_router_scratch_bytes(int N, int M);
 MOE_API int moe_gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias,
                     int N, int K, int M, void* scratch, size_t scratch_bytes, moe_stream_t stream);
 
+/* moe_gemm_router for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference;
+ * its argument list is exactly the reference's gemm_router (src/hip/gemms/gemm_router.hip:184-185),
+ * so it needs no call-site edit.  The fp64 partial sums live in a fixed device array of
+ * MOE_ROUTER_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
+ * ends) instead of a caller buffer; the call allocates nothing.  Same arithmetic and same bits as
+ * moe_gemm_router.  Returns MOE_ERR_LIMIT when the partial sums do not fit the array
+ * (16 * N * M * 8 bytes always fit when N * M <= 131072: 4096 tokens x 32 experts,
+ * 1024 x 128).  All calls on one GPU share the array: calls that overlap on one GPU (two streams,
+ * two host threads) race, calls on one stream do not. */
+#define MOE_ROUTER_STATIC_SCRATCH_BYTES (16u << 20)
+MOE_API size_t moe_gemm_router_static_max_bytes(void);
+MOE_API int moe_gemm_router_static(float* xout, const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias,
+                           int N, int K, int M, moe_stream_t stream);
+
 /* Replaces topk (src/hip/topk.hip:59-72; call site src/forward.cpp:325).  Per token the
  * experts_per_token largest scores in descending order with their indices; equal scores keep
  * the lower expert index first (the order the reference's CPU qsort yields, src/run.cpp:373-404).
