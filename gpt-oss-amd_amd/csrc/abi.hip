@@ -34,6 +34,17 @@ inline bool use_prefill_kernels(int T, int K, int E, int format, unsigned flags)
     return format == MOE_WEIGHTS_MXFP4_TILED ? rows >= 52LL * E : rows >= 448LL * E;
 }
 
+// Bucketing inside the expert kernels instead of a launch of its own: for the weight-streaming
+// kernels, while the assignment list is short enough for one block to scan and buckets mostly fit one
+// 64-token block (a block runs its bucket's token blocks one after the other).
+inline bool use_direct_bucketing(int T, int K, int E, bool prefill, unsigned flags) {
+    if (prefill || (flags & MOE_FLAG_FORCE_BUCKET_LAUNCH)) return false;
+    const long long A = (long long)T * K;
+    if (A > expert_direct_max_assignments() || T > 2048) return false;
+    if (flags & MOE_FLAG_FORCE_DIRECT) return true;
+    return A <= 48LL * E;
+}
+
 // Carves the caller's workspace for moe_block_forward; with base == nullptr only sizes it.
 struct BlockWorkspace {
     double* router_partial;
@@ -379,6 +390,12 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
         rc = launch_router_two_pass(p->t, p->w_router, p->b_router, ws.router_partial, ws.t_bf16, p->topk_v, p->topk_i, T,
                                     H, E, K, 1, stream, timer ? timer->ev[stage++] : nullptr);
         if (rc) return rc;
+    } else if (!strict && router_fused_fits(H)) {
+        // one launch, block per token: the exact pass of the two-pass router applied to every expert
+        rc = launch_router_fused(p->t, p->w_router, p->b_router, ws.t_bf16, p->router_score, p->topk_v, p->topk_i, T, H,
+                                 E, K, 1, stream);
+        if (rc) return rc;
+        if ((rc = mark())) return rc;
     } else {
         const int S = router_segments(T, E, H, strict);
         rc = launch_router_partial(p->t, p->w_router, ws.router_partial, ws.t_bf16, T, H, E, S, stream);
@@ -391,13 +408,18 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     if ((rc = mark())) return rc;
 
     // 2. bucketing + token-block map  (src/forward.cpp:329-376)
+    // Small batches need no bucketing launch: each block of the expert kernels finds its expert's
+    // bucket in topk_i itself and rows are addressed by assignment id (token * K + k).
     const bool prefill = use_prefill_kernels(T, K, E, p->weight_format, p->flags);
+    const bool direct = use_direct_bucketing(T, K, E, prefill, p->flags);
     const int tile_tokens = prefill ? kPrefillTileTokens : kStreamTileTokens;
     const int max_tiles = tile_map_capacity(T * K, E, tile_tokens);  // <= ws.max_tiles (sized for 64)
-    TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles};
-    rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat, ws.slot_of,
-                       map, stream);
-    if (rc) return rc;
+    if (!direct) {
+        TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles};
+        rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat,
+                           ws.slot_of, map, stream);
+        if (rc) return rc;
+    }
     if ((rc = mark())) return rc;
 
     // 3. gate/up GEMM + SwiGLU  (src/forward.cpp:474-479; src/run.cpp:657-689)
@@ -411,11 +433,17 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     g.alpha = p->alpha;
     g.limit = p->swiglu_limit;
     g.format = fmt;
+    if (direct) {
+        g.topk_i = p->topk_i;
+        g.n_assign = T * K;
+        g.assign_div = K;
+        g.n_experts = E;
+    }
 
     // Decode-sized buckets (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of
     // 32 rows each.  Blocks run in rounds of one per CU, so the cheaper choice is the one with the
     // smaller rounds x rows-per-block product; more rows per block also re-read the activations less.
-    const int est_tiles = std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
+    const int est_tiles = direct ? E : std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
     const int kCUs = 256;  // MI355X
     auto pick_consumers = [&](int rows) {
         const int cost10 = ceil_div(ceil_div(rows / 32, 10) * est_tiles, kCUs) * 10;
@@ -484,12 +512,13 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     if ((rc = mark())) return rc;
 
     // 5. weighted combine in ascending expert id (+ residual)  (src/run.cpp:702-712)
+    const int* slot_of = direct ? nullptr : ws.slot_of;  // direct: the row of assignment (t, k) is t * K + k
     if (p->next_norm_out) {
-        rc = launch_combine_norm(ws.y_by_slot, ws.slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x,
+        rc = launch_combine_norm(ws.y_by_slot, slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x,
                                  p->next_norm_weight, p->next_norm_out, T, K, H, stream);
         if (rc != MOE_ERR_LIMIT) return rc ? rc : mark();
     }
-    rc = launch_combine(ws.y_by_slot, ws.slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x, T, K, H, stream);
+    rc = launch_combine(ws.y_by_slot, slot_of, p->topk_i, p->topk_v, p->e_agg, p->residual_x, T, K, H, stream);
     if (rc) return rc;
     if (p->next_norm_out) {  // rows too long for the fused kernel
         rc = launch_rmsnorm(p->next_norm_out, p->residual_x, p->next_norm_weight, T, H, stream);

@@ -5,7 +5,8 @@
 namespace moe {
 
 // The token's K (slot, weight) pairs in ascending expert id (block-uniform: scalar loads and a
-// fully unrolled insertion sort on eight register entries).
+// fully unrolled insertion sort on eight register entries).  slot_of == NULL: rows are stored by
+// assignment, the row of (t, k) is t * K + k.
 MOE_DEVICE void sorted_slots(const int* __restrict__ slot_of, const int* __restrict__ topk_i,
                              const float* __restrict__ topk_v, int t, int K, int (&sl)[8], float (&wt)[8]) {
     int ex[8];
@@ -13,7 +14,7 @@ MOE_DEVICE void sorted_slots(const int* __restrict__ slot_of, const int* __restr
     for (int k = 0; k < 8; ++k) {
         if (k < K) {
             ex[k] = topk_i[(size_t)t * K + k];
-            sl[k] = slot_of[(size_t)t * K + k];
+            sl[k] = slot_of ? slot_of[(size_t)t * K + k] : t * K + k;
             wt[k] = topk_v[(size_t)t * K + k];
         } else {
             ex[k] = 0x7FFFFFFF;
@@ -51,6 +52,48 @@ MOE_DEVICE float4 combine_column(const float4* __restrict__ y, const int (&sl)[8
     return acc;
 }
 
+// Rows stored by assignment (the row of (t, k) is t * K + k): the K rows are known without looking
+// at the routing, so their loads go out together with the loads of the routing itself (one memory
+// round trip instead of two).  The order of the additions is fixed afterwards: the rank of each k by
+// expert id is block-uniform, and rank r is added in step r.
+MOE_DEVICE float4 combine_column_by_assignment(const float4* __restrict__ y, const int* __restrict__ topk_i,
+                                               const float* __restrict__ topk_v, int t, int K, int H4, int c) {
+    float4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        if (k < K) v[k] = y[((size_t)t * K + k) * H4 + c];
+    int ex[8];
+    float wt[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        ex[k] = k < K ? topk_i[(size_t)t * K + k] : 0x7FFFFFFF;
+        wt[k] = k < K ? topk_v[(size_t)t * K + k] : 0.f;
+    }
+    int rank[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        rank[k] = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) rank[k] += (ex[j] < ex[k] || (ex[j] == ex[k] && j < k)) ? 1 : 0;
+    }
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        if (r < K) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                if (k < K && rank[k] == r) {  // block-uniform
+                    acc.x = fmaf(v[k].x, wt[k], acc.x);
+                    acc.y = fmaf(v[k].y, wt[k], acc.y);
+                    acc.z = fmaf(v[k].z, wt[k], acc.z);
+                    acc.w = fmaf(v[k].w, wt[k], acc.w);
+                }
+            }
+        }
+    }
+    return acc;
+}
+
 // e_agg[t,:] = sum over the token's K experts, visited in ASCENDING EXPERT ID, of
 // y_by_slot[slot,:] * weight, each step one fused multiply-add — the order and rounding of the
 // reference CPU loop (src/run.cpp:645-706).  Replaces the atomicAdd scatter of
@@ -64,10 +107,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const float4* __restrict__
     const int t = blockIdx.y;
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= H4) return;
-    int sl[8];
-    float wt[8];
-    sorted_slots(slot_of, topk_i, topk_v, t, K, sl, wt);
-    const float4 acc = combine_column(y, sl, wt, K, H4, c);
+    float4 acc;
+    if (slot_of) {
+        int sl[8];
+        float wt[8];
+        sorted_slots(slot_of, topk_i, topk_v, t, K, sl, wt);
+        acc = combine_column(y, sl, wt, K, H4, c);
+    } else {
+        acc = combine_column_by_assignment(y, topk_i, topk_v, t, K, H4, c);
+    }
     e_agg[(size_t)t * H4 + c] = acc;
     if (residual_x) {
         float4 r = residual_x[(size_t)t * H4 + c];

@@ -61,8 +61,9 @@ MOE_DEVICE void load_bias(const ExpertGemmArgs& a, int e, int group, int r0, uin
     for (int r = 0; r < R; ++r) raw[r] = *reinterpret_cast<const uint2*>(bias + 4 * r);
 }
 
-template <int R, int NT, int EPI>
-MOE_DEVICE void stream_epilogue(const ExpertGemmArgs& a, const f32x4 (&acc)[R][NT], int e, int row0, int nrows,
+// slot_of_row(i): output row (slot) of bucket row i of the token block.
+template <int R, int NT, int EPI, class SlotFn>
+MOE_DEVICE void stream_epilogue(const ExpertGemmArgs& a, const f32x4 (&acc)[R][NT], int e, SlotFn slot_of_row, int nrows,
                                 int group, int r0, const uint2 (&bias_raw)[R]) {
     const int lane = threadIdx.x & 63;
     const int q = lane & 15;
@@ -81,7 +82,7 @@ MOE_DEVICE void stream_epilogue(const ExpertGemmArgs& a, const f32x4 (&acc)[R][N
     for (int t = 0; t < NT; ++t) {
         const int idx = t * 16 + q;
         if (idx >= nrows) continue;
-        const size_t slot = (size_t)row0 + idx;
+        const size_t slot = (size_t)slot_of_row(idx);
         if constexpr (EPI == EPI_SWIGLU_BF16 || EPI == EPI_SWIGLU_F32) {
             const int I = a.rows / 2;
             float h[R][2];
@@ -356,7 +357,7 @@ MOE_DEVICE void stream_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int ro
 
     uint2 bias_raw[R];
     load_bias<R>(a, e, group, r0, bias_raw);
-    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0, bias_raw);
+    stream_epilogue<R, NT, EPI>(a, acc, e, [&](int i) { return row0 + i; }, nrows, group, r0, bias_raw);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -392,8 +393,9 @@ MOE_DEVICE int ws_chunk(int j, int g) {  // chunk holding the operand of MFMA st
     return (FMT == FMT_BF16) ? 8 * (j >> 1) + 2 * g + (j & 1) : 4 * g + j;
 }
 
-template <int FMT, int NT, int PROD>
-MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int nrows, int p) {
+// act_row(i): row of a.act that holds bucket row i of the token block (i < nrows).
+template <int FMT, int NT, int PROD, class RowFn>
+MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row, int nrows, int p) {
     constexpr int BP = 4 / PROD;  // four-row blocks of a token tile moved by this wave
     constexpr int Q = BP * NT;    // direct-to-LDS loads per stage issued by this wave
     const int lane = threadIdx.x & 63;
@@ -416,8 +418,7 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int idx = min(t * 16 + q, nrows - 1);
-            const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
-            row[t][ii] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
+            row[t][ii] = reinterpret_cast<const uint8_t*>(a.act + (size_t)act_row(idx) * K);
         }
     }
     auto issue = [&](int s) {
@@ -455,8 +456,12 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, int row0, int
     wait_vmcnt<0>();  // nothing may still be writing this block's LDS when the wave ends
 }
 
-template <int FMT, int NT, int EPI>
-MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, int row0, int nrows, int unit,
+// slot_of_row(i): output row of bucket row i.  PRE: one more barrier comes first, right after the
+// first weight loads have been issued (the kernel that finds the bucket itself completes the bucket
+// list behind that barrier; the consumers need the list only in their epilogue, so their weights are
+// already on the way while the producers read it).
+template <int FMT, int NT, int EPI, bool PRE = false, class SlotFn>
+MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows, int unit,
                             bool active) {
     constexpr int R = 2;
     const int lane = threadIdx.x & 63;
@@ -465,7 +470,7 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     const int K = a.K;
     const int n_stages = ceil_div(K, kStageElems);
     if (!active) {
-        for (int i = 0; i <= n_stages; ++i) __syncthreads();
+        for (int i = 0; i <= n_stages + (PRE ? 1 : 0); ++i) __syncthreads();
         return;
     }
     const int group = unit >> 1;
@@ -510,6 +515,7 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         };
 #pragma unroll
         for (int i = 0; i < DP - 1; ++i) load_a(i, i);
+        if constexpr (PRE) __syncthreads();
         __syncthreads();
         // one stage = two pairs; `ss` (stage parity) fixes the ring slots at compile time
         auto stage = [&](auto ss_tag, int st) {
@@ -593,6 +599,7 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         load_scales(sw_cur, 0);
 #pragma unroll
         for (int i = 0; i < D - 1; ++i) load_a(i, i);
+        if constexpr (PRE) __syncthreads();
         __syncthreads();
         // stage st, the i-th of its group of four (i fixes ring slot and scale byte at compile time)
         auto stage = [&](auto i_tag, int st) {
@@ -635,43 +642,149 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         if (tail > 1) stage(std::integral_constant<int, 1>{}, 4 * full_quads + 1);
         if (tail > 2) stage(std::integral_constant<int, 2>{}, 4 * full_quads + 2);
     }
-    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, group, r0, bias_raw);
+    stream_epilogue<R, NT, EPI>(a, acc, e, slot_of_row, nrows, group, r0, bias_raw);
 }
 
+// One token block: the producer or consumer role of this wave, for the block's token-tile count.
+template <int FMT, int EPI, int CONS, int PROD, bool PRE = false, class RowFn, class SlotFn>
+MOE_DEVICE void ws_token_block(const ExpertGemmArgs& a, uint8_t* lds, int wave, int unit, bool active, int e,
+                               RowFn act_row, SlotFn slot_of_row, int nrows) {
+    const int nt = (nrows + 15) >> 4;  // block-uniform
+    if (wave >= CONS) {
+        const int p = wave - CONS;
+        if constexpr (PRE) __syncthreads();  // no direct-to-LDS load is in flight yet
+        if (nt == 4) ws_producer<FMT, 4, PROD>(a, lds, act_row, nrows, p);
+        else if (nt == 3) ws_producer<FMT, 3, PROD>(a, lds, act_row, nrows, p);
+        else if (nt == 2) ws_producer<FMT, 2, PROD>(a, lds, act_row, nrows, p);
+        else ws_producer<FMT, 1, PROD>(a, lds, act_row, nrows, p);
+    } else {
+        if (nt == 4) ws_consumer<FMT, 4, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
+        else if (nt == 3) ws_consumer<FMT, 3, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
+        else if (nt == 2) ws_consumer<FMT, 2, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
+        else ws_consumer<FMT, 1, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
+    }
+}
+
+// Linear block index -> (token block or expert, row block).  Workgroups go to the eight XCDs
+// round-robin by linear index; with xcd_tiles all row blocks of an item run on one XCD (its
+// activations enter one L2 once), otherwise they are spread over all of them.
+MOE_DEVICE void ws_block_coords(const ExpertGemmArgs& a, int& item, int& rb) {
+    const int n_rb = a.row_blocks;
+    item = a.xcd_tiles ? ((blockIdx.x >> 3) / n_rb) * 8 + (blockIdx.x & 7) : blockIdx.x / n_rb;
+    rb = a.xcd_tiles ? (blockIdx.x >> 3) % n_rb : blockIdx.x % n_rb;
+}
+
+// the row units of the weight matrix are spread evenly over the row blocks
+MOE_DEVICE void ws_row_unit(const ExpertGemmArgs& a, int rb, int wave, int& unit, bool& active) {
+    const int units = a.rows / 32;
+    const int u0 = (int)((long long)rb * units / a.row_blocks);
+    const int u1 = (int)((long long)(rb + 1) * units / a.row_blocks);
+    unit = u0 + wave;
+    active = unit < u1;
+}
+
+// Token blocks from the tile map written by the bucketing kernel.
 // grid = row blocks x token blocks (padded to a multiple of 8), block = 64 (CONS + PROD); one block per CU: twelve
 // waves leave 168 registers per lane, fourteen leave 128.
 template <int FMT, int EPI, int CONS, int PROD>
 __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) void expert_stream_ws_kernel(ExpertGemmArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kWsRing * kLdsStageBytes];
-    // Linear block index -> (token block, row block).  Workgroups go to the eight XCDs round-robin by
-    // linear index; with a.xcd_tiles all row blocks of a token block run on one XCD (its activations
-    // enter one L2 once), otherwise they are spread over all of them.
-    const int n_rb = a.row_blocks;
-    const int tile = a.xcd_tiles ? ((blockIdx.x >> 3) / n_rb) * 8 + (blockIdx.x & 7) : blockIdx.x / n_rb;
-    const int rb = a.xcd_tiles ? (blockIdx.x >> 3) % n_rb : blockIdx.x % n_rb;
+    int tile, rb;
+    ws_block_coords(a, tile, rb);
     if (tile >= *a.n_tiles) return;  // block-uniform
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int e = a.tile_expert[tile];
     const int row0 = a.tile_row0[tile];
     const int nrows = a.tile_rows[tile];
-    const int nt = (nrows + 15) >> 4;  // block-uniform
-    if (wave >= CONS) {
-        const int p = wave - CONS;
-        if (nt == 4) ws_producer<FMT, 4, PROD>(a, lds, row0, nrows, p);
-        else if (nt == 3) ws_producer<FMT, 3, PROD>(a, lds, row0, nrows, p);
-        else if (nt == 2) ws_producer<FMT, 2, PROD>(a, lds, row0, nrows, p);
-        else ws_producer<FMT, 1, PROD>(a, lds, row0, nrows, p);
-    } else {
-        // the row units of the weight matrix are spread evenly over the gridDim.x row blocks
-        const int units = a.rows / 32;
-        const int u0 = (int)((long long)rb * units / n_rb);
-        const int u1 = (int)((long long)(rb + 1) * units / n_rb);
-        const int unit = u0 + wave;
-        const bool active = unit < u1;
-        if (nt == 4) ws_consumer<FMT, 4, EPI>(a, lds, e, row0, nrows, unit, active);
-        else if (nt == 3) ws_consumer<FMT, 3, EPI>(a, lds, e, row0, nrows, unit, active);
-        else if (nt == 2) ws_consumer<FMT, 2, EPI>(a, lds, e, row0, nrows, unit, active);
-        else ws_consumer<FMT, 1, EPI>(a, lds, e, row0, nrows, unit, active);
+    int unit;
+    bool active;
+    ws_row_unit(a, rb, wave, unit, active);
+    ws_token_block<FMT, EPI, CONS, PROD>(
+        a, lds, wave, unit, active, e, [&](int i) { return a.gather ? a.tokens_flat[row0 + i] : row0 + i; },
+        [&](int i) { return row0 + i; }, nrows);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same expert GEMM without a bucketing launch in front of it, for batches of at most
+// kDirectMaxAssign assignments (tokens x experts per token).  A block is one (expert, row block)
+// pair, known from the block index alone, and finds the expert's bucket itself: every wave compares
+// chunks of 64 consecutive assignments of topk_i with the expert id, the per-chunk match counts go
+// through LDS, one wave-wide prefix sum gives every chunk its offset, and the matching assignment
+// ids (token * experts_per_token + k, ascending: the bucket order of bucket_kernel) land in an LDS
+// list.  The block then runs the bucket's token blocks of up to 64 rows one after the other.
+// Rows are addressed by assignment id: the activation row of assignment s is s / assign_div (gate/up
+// launch: the token's row) or s itself (down launch), and the output row is s.
+// grid = row blocks x experts (padded to a multiple of 8), block = 64 (CONS + PROD).
+// ---------------------------------------------------------------------------------------------
+constexpr int kDirectMaxAssign = 4096;  // 64 chunks of 64: one lane per chunk in the prefix sum
+constexpr int kDirectMaxRows = 2048;    // longest bucket the LDS list holds
+
+template <int FMT, int EPI, int CONS, int PROD>
+__global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) void expert_stream_direct_kernel(ExpertGemmArgs a) {
+    constexpr int WAVES = CONS + PROD;
+    constexpr int P = (64 + WAVES - 1) / WAVES;  // chunks per wave
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kWsRing * kLdsStageBytes];
+    __shared__ int bucket[kDirectMaxRows];
+    __shared__ int chunk_cnt[64];
+    int e, rb;
+    ws_block_coords(a, e, rb);
+    if (e >= a.n_experts) return;  // block-uniform (grid padding)
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_chunks = (a.n_assign + 63) >> 6;
+    int unit;
+    bool active;
+    ws_row_unit(a, rb, wave, unit, active);
+    int n_bucket;
+    {
+        // this wave's chunks of the assignment list
+        int ids[P];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int s = (p * WAVES + wave) * 64 + lane;
+            ids[p] = s < a.n_assign ? a.topk_i[s] : -1;
+        }
+        unsigned long long match[P];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int c = p * WAVES + wave;
+            match[p] = __ballot(ids[p] == e);
+            if (lane == 0 && c < n_chunks) chunk_cnt[c] = __popcll(match[p]);
+        }
+        __syncthreads();
+        // inclusive prefix sum of the chunk counts over the wave's lanes
+        uint32_t incl = lane < n_chunks ? (uint32_t)chunk_cnt[lane] : 0u;
+#define MOE_STEP(C, M) incl += dpp_move<C, M>(0u, incl);
+        MOE_DPP_STEPS(MOE_STEP)
+#undef MOE_STEP
+        n_bucket = min((int)__builtin_amdgcn_readlane(incl, 63), kDirectMaxRows);
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int c = p * WAVES + wave;
+            if (c < n_chunks) {  // wave-uniform
+                const int base = (int)__builtin_amdgcn_readlane(incl, c) - __popcll(match[p]);
+                const int dst = base + __popcll(match[p] & ((1ull << lane) - 1ull));
+                if (ids[p] == e && dst < kDirectMaxRows) bucket[dst] = c * 64 + lane;
+            }
+        }
+        // the barrier that completes the list is the first one of the token block below
+    }
+    if (n_bucket == 0) return;
+    // token of assignment s = s / assign_div, as a float multiplication (exact for s < 4096, assign_div <= 8)
+    const float inv_div = 1.0f / (float)a.assign_div;
+    auto token_of = [&](int s) { return (int)(((float)s + 0.5f) * inv_div); };
+    // The first token block takes the bucket's remainder (1..64 rows, any tile count) in straight-line
+    // code; what is left are whole blocks of 64 rows, run by a loop that holds the four-tile variant
+    // only (a loop around all tile-count variants costs every variant 30 registers per lane).
+    const int first = n_bucket - ((n_bucket - 1) & ~63);
+    ws_token_block<FMT, EPI, CONS, PROD, true>(
+        a, lds, wave, unit, active, e, [&](int i) { return a.gather ? token_of(bucket[i]) : bucket[i]; },
+        [&](int i) { return bucket[i]; }, first);
+    for (int row0 = first; row0 < n_bucket; row0 += 64) {
+        auto act_row = [&](int i) { return a.gather ? token_of(bucket[row0 + i]) : bucket[row0 + i]; };
+        auto slot_of_row = [&](int i) { return bucket[row0 + i]; };
+        if (wave >= CONS) ws_producer<FMT, 4, PROD>(a, lds, act_row, 64, wave - CONS);
+        else ws_consumer<FMT, 4, EPI>(a, lds, e, slot_of_row, 64, unit, active);
     }
 }
 
@@ -858,7 +971,7 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     }
     uint2 bias_raw[R];
     load_bias<R>(a, e, unit, 0, bias_raw);
-    stream_epilogue<R, NT, EPI>(a, acc, e, row0, nrows, unit, 0, bias_raw);
+    stream_epilogue<R, NT, EPI>(a, acc, e, [&](int i) { return row0 + i; }, nrows, unit, 0, bias_raw);
 }
 
 template <int FMT, int NT, int EPI, int WAVES>
@@ -916,7 +1029,18 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
         dim3 grid(ceil_div(units, 4), max(1, ceil_div(a.max_rows_hint, 64)), a.work_count);
         hipLaunchKernelGGL((expert_stream_queue_kernel<FMT, R, EPI>), grid, dim3(256), 0, stream, a);
     } else if constexpr (EPI == EPI_SWIGLU_BF16 || EPI == EPI_ROWS_F32) {
-        if (a.waves_per_block == 16) {
+        if (a.topk_i) {  // bucketing inside the expert kernel
+            if (a.n_assign > kDirectMaxAssign || a.assign_div <= 0 || a.assign_div > 8 || a.n_experts <= 0) return MOE_ERR_LIMIT;
+            ExpertGemmArgs b = a;
+            const int cons = a.waves_per_block == 1 ? 12 : 10;
+            b.row_blocks = max(a.row_blocks, ceil_div(a.rows / 32, cons));
+            dim3 grid(ceil_div(a.n_experts, 8) * 8 * b.row_blocks);
+            if (cons == 12) {
+                hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, b);
+            } else {
+                hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, b);
+            }
+        } else if (a.waves_per_block == 16) {
             ExpertGemmArgs b = a;
             b.row_blocks = ceil_div(a.rows / 64, 4);
             dim3 grid(ceil_div(a.max_tiles, 8) * 8 * b.row_blocks);  // every XCD gets whole token blocks
@@ -952,6 +1076,8 @@ int launch_fmt(const ExpertGemmArgs& a, int epi, hipStream_t stream) {
 }
 
 }  // namespace
+
+int expert_direct_max_assignments() { return kDirectMaxAssign; }
 
 // epi: 0 fused gate/up (bf16 SwiGLU out), 1 fused down (fp32 rows per slot), 2 gate/up with fp32
 // in/out, 3 down with fp32 in and atomic scatter.  Token blocks hold at most 64 rows.

@@ -14,6 +14,11 @@ int launch_router_finalize(const double* partial, int S, const float* scores_in,
                            float* scores_out, float* topk_v, int* topk_i, int T, int E, int K, int do_topk,
                            int do_softmax, hipStream_t stream);
 int launch_softmax_rows(float* x, int B, int size, hipStream_t stream);
+// Whole router in one launch (block per token): logits as the exact pass of the two-pass router,
+// top-k, softmax, the bf16 activation copy and, if scores_out is not NULL, the score matrix.
+bool router_fused_fits(int H);
+int launch_router_fused(const float* x, const uint16_t* w, const uint16_t* bias, uint16_t* x_bf16, float* scores_out,
+                        float* topk_v, int* topk_i, int T, int H, int E, int K, int do_softmax, hipStream_t stream);
 // Two-pass router (fp32 screening of all experts, exact scores of the candidates): same top-k and
 // softmax as partial + finalize.  `scratch` holds router_screen_bytes(); `between`, if not NULL, is
 // recorded after the first pass.
@@ -52,6 +57,11 @@ struct ExpertGemmArgs {
     const int* tokens_flat;     // slot row -> token id
     const float* weights_flat;  // slot row -> router weight (scatter epilogue)
     int gather;                 // 1: activation row = tokens_flat[slot row]; 0: slot row itself
+    const int* topk_i;          // non-null: no tile map, the kernel buckets the [n_assign] expert ids itself and
+                                // addresses rows by assignment id (token * experts_per_token + k)
+    int n_assign;               // tokens x experts per token
+    int assign_div;             // activation row of assignment s: s / assign_div when gather, else s
+    int n_experts;
     const int* work_queue;      // non-null: (expert, row_offset, row_count) triples instead of the tile map
     int work_start, work_count, max_rows_hint;
     const int* tile_expert;
@@ -75,6 +85,7 @@ struct ExpertGemmArgs {
                                 // 128-token blocks).  Ignored by the work-queue entries.
 };
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
+int expert_direct_max_assignments();
 
 // ---- combine.hip -------------------------------------------------------------------------------
 int launch_combine(const float* y_by_slot, const int* slot_of, const int* topk_i, const float* topk_v,

@@ -483,20 +483,22 @@ __global__ __launch_bounds__(256) void router_screen_kernel(const float* __restr
     }
 }
 
-// Exact logits of four experts for one token, by one wave: fp32 products, fp64 sums
+// Exact logits of NE experts for one token, by one wave: fp32 products, fp64 sums
 // (src/run.cpp:341-354).  Lane l takes float4 number l, l + 64, ... of the token's activations in
-// ascending order; the lanes' sums are combined by wave_sum's fixed tree.  The trip count is the
-// same for every lane (a lane past the end multiplies zeros), so that the loads of several
-// iterations can be in flight together.  Every lane returns all four totals.
-MOE_DEVICE void exact_dots4(const float* __restrict__ x_row, const uint16_t* __restrict__ w, const int (&e)[4], int H,
-                            int lane, double (&total)[4]) {
+// ascending order; the lanes' sums are combined by wave_sum's fixed tree, so a logit does not depend
+// on NE or on which other experts share the call.  The trip count is the same for every lane (a
+// lane past the end multiplies zeros), so that the loads of several iterations can be in flight
+// together.  Every lane returns all NE totals.
+template <int NE>
+MOE_DEVICE void exact_dots(const float* __restrict__ x_row, const uint16_t* __restrict__ w, const int (&e)[NE], int H,
+                           int lane, double (&total)[NE]) {
     const int n4 = H >> 2;
     const int trips = ceil_div(n4, 64);
     const float4* xrow = reinterpret_cast<const float4*>(x_row);
-    const uint2* wrow[4];
-    double acc[4];
+    const uint2* wrow[NE];
+    double acc[NE];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NE; ++i) {
         wrow[i] = reinterpret_cast<const uint2*>(w + (size_t)e[i] * H);
         acc[i] = 0.0;
     }
@@ -505,11 +507,11 @@ MOE_DEVICE void exact_dots4(const float* __restrict__ x_row, const uint16_t* __r
         const bool live = lane + 64 * j < n4;
         const int i4 = min(lane + 64 * j, n4 - 1);
         const float4 xv = xrow[i4];
-        uint2 wb[4];
+        uint2 wb[NE];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) wb[i] = wrow[i][i4];
+        for (int i = 0; i < NE; ++i) wb[i] = wrow[i][i4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NE; ++i) {
             if (!live) wb[i] = make_uint2(0u, 0u);  // zero products leave the sum unchanged
             acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x << 16), xv.x);
             acc[i] += (double)__fmul_rn(__uint_as_float(wb[i].x & 0xFFFF0000u), xv.y);
@@ -518,7 +520,124 @@ MOE_DEVICE void exact_dots4(const float* __restrict__ x_row, const uint16_t* __r
         }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) total[i] = wave_sum(acc[i]);
+    for (int i = 0; i < NE; ++i) total[i] = wave_sum(acc[i]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Whole router in one launch for batches too small for the two-pass router to pay: one block per
+// token.  The block stages the token's activation row in LDS (and writes its row of the bf16 copy
+// that the expert GEMMs consume); wave w scores experts NE*w .. NE*w + NE-1 (then NE*(w + waves) ..,
+// if there are more) with the arithmetic and the order of additions of exact_dots — the same logits, bit for bit,
+// as the exact pass of the two-pass router — and leaves them in LDS; wave 0 then runs top-k and
+// softmax and writes the score row if the caller wants it.
+// All loads of a wave's first pass (the activation piece it stages, its two router rows) are issued
+// before anything waits, so a block costs one memory round trip plus the arithmetic.
+// grid = T, block = 64 * waves, dynamic LDS = (H + E) floats; H <= 256 * kFusedTrips.  NE experts per
+// wave and pass: two with up to 16 waves (128 registers per lane hold the loads of two rows), four
+// with up to 8 waves.
+// ---------------------------------------------------------------------------------------------
+constexpr int kFusedTrips = 12;  // rows of up to 3072 values
+
+template <int NE>
+__global__ __launch_bounds__(NE == 2 ? 1024 : 512) void router_fused_kernel(const float* __restrict__ x, const uint16_t* __restrict__ w,
+                                                            const uint16_t* __restrict__ bias,
+                                                            uint16_t* __restrict__ x_bf16,
+                                                            float* __restrict__ scores_out, float* __restrict__ topk_v,
+                                                            int* __restrict__ topk_i, int H, int E, int K,
+                                                            int do_softmax) {
+    extern __shared__ __attribute__((aligned(16))) float fused_lds[];
+    float4* xs = reinterpret_cast<float4*>(fused_lds);  // [H / 4]
+    float* sc = fused_lds + H;                           // [E]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = blockDim.x >> 6;
+    const int t = blockIdx.x;
+    const int n4 = H >> 2;
+    const float4* xr = reinterpret_cast<const float4*>(x + (size_t)t * H);
+    const int n_groups = ceil_div(E, NE);
+
+    // activation row: thread i stages float4 number i, i + blockDim, ...
+    constexpr int STG = NE == 2 ? 1 : 2;  // enough for a full-size block; smaller blocks take the loops below
+    float4 xv_st[STG];
+#pragma unroll
+    for (int i = 0; i < STG; ++i) {
+        const int c = threadIdx.x + i * blockDim.x;
+        xv_st[i] = xr[min(c, n4 - 1)];
+    }
+    // per-lane element index of trip j, clamped into the row; as 32-bit byte offsets next to
+    // wave-uniform row bases the loads need no per-lane 64-bit addresses
+    uint32_t idx[kFusedTrips];
+#pragma unroll
+    for (int j = 0; j < kFusedTrips; ++j) idx[j] = (uint32_t)min(lane + 64 * j, n4 - 1);
+    uint2 wb[kFusedTrips][NE];
+    auto load_rows = [&](int grp) {
+#pragma unroll
+        for (int i = 0; i < NE; ++i) {
+            const char* wrow = reinterpret_cast<const char*>(w + (size_t)min(grp * NE + i, E - 1) * H);
+#pragma unroll
+            for (int j = 0; j < kFusedTrips; ++j) wb[j][i] = *reinterpret_cast<const uint2*>(wrow + (size_t)(idx[j] * 8u));
+        }
+    };
+    if (wave < n_groups) load_rows(wave);
+    for (int c = threadIdx.x + STG * blockDim.x; c < n4; c += blockDim.x) xs[c] = xr[c];  // blocks with few waves
+#pragma unroll
+    for (int i = 0; i < STG; ++i) {
+        const int c = threadIdx.x + i * blockDim.x;
+        if (c < n4) {
+            xs[c] = xv_st[i];
+            if (x_bf16)
+                reinterpret_cast<uint2*>(x_bf16 + (size_t)t * H)[c] =
+                    make_uint2(pack_bf16x2(xv_st[i].x, xv_st[i].y), pack_bf16x2(xv_st[i].z, xv_st[i].w));
+        }
+    }
+    if (x_bf16)
+        for (int c = threadIdx.x + STG * blockDim.x; c < n4; c += blockDim.x) {
+            const float4 v = xr[c];
+            reinterpret_cast<uint2*>(x_bf16 + (size_t)t * H)[c] = make_uint2(pack_bf16x2(v.x, v.y), pack_bf16x2(v.z, v.w));
+        }
+    __syncthreads();
+    auto score_group = [&](int grp) {
+        double acc[NE];
+#pragma unroll
+        for (int i = 0; i < NE; ++i) acc[i] = 0.0;
+#pragma unroll
+        for (int j = 0; j < kFusedTrips; ++j) {
+            const bool live = lane + 64 * j < n4;
+            const float4 xv = xs[idx[j]];
+#pragma unroll
+            for (int i = 0; i < NE; ++i) {
+                const uint2 wv = live ? wb[j][i] : make_uint2(0u, 0u);  // zero products leave the sum unchanged
+                acc[i] += (double)__fmul_rn(__uint_as_float(wv.x << 16), xv.x);
+                acc[i] += (double)__fmul_rn(__uint_as_float(wv.x & 0xFFFF0000u), xv.y);
+                acc[i] += (double)__fmul_rn(__uint_as_float(wv.y << 16), xv.z);
+                acc[i] += (double)__fmul_rn(__uint_as_float(wv.y & 0xFFFF0000u), xv.w);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NE; ++i) {
+            const double total = wave_sum(acc[i]);
+            const int e = grp * NE + i;
+            if (lane == 0 && e < E) sc[e] = (float)total + bf16_bits_to_f32(bias[e]);
+        }
+    };
+    // the usual case, one group per wave, is straight-line code (a loop here makes the compiler hoist
+    // every trip's address arithmetic out of it and hold it in registers)
+    if (wave < n_groups) score_group(wave);
+    if (n_groups > n_waves) {
+#pragma nounroll
+        for (int grp = wave + n_waves; grp < n_groups; grp += n_waves) {
+            load_rows(grp);
+            score_group(grp);
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    if (scores_out)
+        for (int e = lane; e < E; e += 64) scores_out[(size_t)t * E + e] = sc[e];
+    float my_v;
+    int my_i;
+    select_topk(sc, E, K, lane, my_v, my_i);
+    write_topk(my_v, my_i, K, lane, do_softmax, topk_v + (size_t)t * K, topk_i + (size_t)t * K);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -639,7 +758,7 @@ __global__ __launch_bounds__(256, 4) void router_refine_kernel(const float* __re
         double total[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) e[i] = __builtin_amdgcn_readfirstlane(cand[min(c0 + i, n_cand - 1)]);
-        exact_dots4(x_row, w, e, H, lane, total);
+        exact_dots<4>(x_row, w, e, H, lane, total);
         if (lane == 0) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) exact[e[i]] = (float)total[i] + bf16_bits_to_f32(bias[e[i]]);
@@ -778,6 +897,25 @@ int launch_router_finalize(const double* partial, int S, const float* scores_in,
     hipLaunchKernelGGL(router_finalize_kernel, dim3(ceil_div(T, 4)), dim3(256), (size_t)4 * E * sizeof(float),
                        stream, partial, S, scores_in, bias, scores_out, topk_v, topk_i, T, E, K, do_topk,
                        do_softmax);
+    return launch_status();
+}
+
+// Rows the fused router can take (all of a wave's loads are held in registers at once).
+bool router_fused_fits(int H) { return H % 4 == 0 && H <= 256 * kFusedTrips; }
+
+// Up to 32 experts: two per wave, up to 16 waves (the shortest critical path per token); beyond: four
+// per wave, 8 waves, as many passes as that takes.
+int launch_router_fused(const float* x, const uint16_t* w, const uint16_t* bias, uint16_t* x_bf16, float* scores_out,
+                        float* topk_v, int* topk_i, int T, int H, int E, int K, int do_softmax, hipStream_t stream) {
+    if (!router_fused_fits(H)) return MOE_ERR_LIMIT;
+    const size_t lds = (size_t)(H + E) * sizeof(float);
+    if (E <= 32) {
+        hipLaunchKernelGGL(router_fused_kernel<2>, dim3(T), dim3(64 * min(16, ceil_div(E, 2))), lds, stream, x, w, bias,
+                           x_bf16, scores_out, topk_v, topk_i, H, E, K, do_softmax);
+    } else {
+        hipLaunchKernelGGL(router_fused_kernel<4>, dim3(T), dim3(64 * min(8, ceil_div(E, 4))), lds, stream, x, w, bias,
+                           x_bf16, scores_out, topk_v, topk_i, H, E, K, do_softmax);
+    }
     return launch_status();
 }
 

@@ -255,7 +255,11 @@ enum {
     MOE_FLAG_ROUTER_STRICT_ORDER = 1u, /* accumulate each router dot product in one sequential
                                           pass over k, exactly the order of src/run.cpp:348-351 */
     MOE_FLAG_FORCE_STREAM = 2u,        /* always use the weight-streaming expert kernels */
-    MOE_FLAG_FORCE_TILED = 4u          /* always use the LDS-tiled expert kernels */
+    MOE_FLAG_FORCE_TILED = 4u,         /* always use the LDS-tiled expert kernels */
+    MOE_FLAG_FORCE_DIRECT = 8u,        /* weight-streaming kernels: bucket inside the expert kernels whenever
+                                          the batch allows it (n_tokens * experts_per_token <= 4096,
+                                          n_tokens <= 2048), however long the buckets */
+    MOE_FLAG_FORCE_BUCKET_LAUNCH = 16u /* always run the bucketing kernel and its token-block map */
 };
 
 MOE_API size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int intermediate_dim, int n_experts,

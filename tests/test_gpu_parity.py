@@ -210,8 +210,13 @@ def test_block_small(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
     # strict router order gives the same routing, and the whole call is deterministic
     y2, ti2, tv2 = blk.forward(x, flags=pkg.MOE_FLAG_ROUTER_STRICT_ORDER)
     assert torch.equal(ti2, ti) and torch.equal(y2, y) and torch.equal(tv2, tv)
-    # both kernel families on every shape, whichever the size rule picked above
-    for name, flag in (("64-token blocks", pkg.MOE_FLAG_FORCE_STREAM), ("128-token blocks", pkg.MOE_FLAG_FORCE_TILED)):
+    # both kernel families on every shape, and the streaming family with either way of bucketing
+    # (inside the expert kernels / by the bucketing launch), whichever the size rule picked above
+    for name, flag in (("64-token blocks, bucketing in the expert kernels",
+                        pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT),
+                       ("64-token blocks, bucketing launch",
+                        pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH),
+                       ("128-token blocks", pkg.MOE_FLAG_FORCE_TILED)):
         yf, tif, _ = blk.forward(x, flags=flag)
         errf = hostgen.rel_err(yf.cpu().numpy(), ref_y)
         say("  %s: rel err %.3e" % (name, errf))
@@ -279,7 +284,8 @@ def test_block_random_shapes(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
     x = wl.make_device_input(shape, table, dev)
     hw = hostgen.host_layer(oracle, wl, shape)
     ref_y, ref_i, ref_v, _ = hostgen.oracle_block(oracle, shape, hw, hostgen.host_input(oracle, wl, shape))
-    for flags in (0, pkg.MOE_FLAG_FORCE_STREAM, pkg.MOE_FLAG_FORCE_TILED):
+    for flags in (0, pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT,
+                  pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH, pkg.MOE_FLAG_FORCE_TILED):
         y, ti, tv = blk.forward(x, flags=flags)
         torch.cuda.synchronize()
         assert np.array_equal(ti.cpu().numpy(), ref_i), flags
