@@ -81,6 +81,7 @@ SIGNATURES = {
     "moe_softmax": (_i, [_vp, _i, _i, _vp]),
     "moe_bucket_by_expert": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "moe_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "moe_scatter_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "moe_build_work_queue": (_i, [_vp, _i, _vp, _vp, _vp]),
     "moe_mlp1_swiglu": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _ll, _ll, _f, _f, _i, _i, _vp]),
     "moe_mlp2_scatter": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _ll, _ll, _i, _i, _vp]),
@@ -183,6 +184,11 @@ def bucket_by_expert(topk_i, topk_v, B, K, E, expert_offsets, tokens_flat, weigh
 def gather_rows(X, idx, Y, rows, H, stream=None):
     """src/hip/scheduler.hip:63-85."""
     _check("moe_gather_rows", _lib.moe_gather_rows(_ptr(X), _ptr(idx), _ptr(Y), rows, H, _stream(stream)))
+
+
+def scatter_rows(Y, idx, X, rows, H, stream=None):
+    """X[idx[row], :] = Y[row, :] (inverse of gather_rows)."""
+    _check("moe_scatter_rows", _lib.moe_scatter_rows(_ptr(Y), _ptr(idx), _ptr(X), rows, H, _stream(stream)))
 
 
 def build_work_queue(expert_offsets, E, work_queue, work_count, stream=None):

@@ -13,7 +13,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmoe_gfx950.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.environ.get("HIPCC", os.path.join(ROCM, "bin", "hipcc"))
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
@@ -57,8 +58,31 @@ def up_to_date():
     return all(os.path.getmtime(p) <= t for p in sources() + headers() + [os.path.abspath(__file__)])
 
 
+HOST_DIR = os.path.join(HERE, "host")
+HOST_BIN_DIR = os.path.join(HOST_DIR, "bin")
+HOST_PROGRAMS = ["moe_stack_main", "example_layer_loop"]
+
+
+def build_host_programs():
+    """The C++ host side (layer loop, forward(), decode loop) as programs linked against the library:
+    compiled here so that the GPU box only has to run them.  Plain C++ against the HIP runtime API."""
+    os.makedirs(HOST_BIN_DIR, exist_ok=True)
+    out = []
+    for name in HOST_PROGRAMS:
+        exe = os.path.join(HOST_BIN_DIR, name)
+        cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__",
+               "-I" + os.path.join(ROCM, "include"), os.path.join(HOST_DIR, name + ".cpp"), "-o", exe, "-L" + HERE,
+               "-lmoe_gfx950", "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN/../..",
+               "-Wl,-rpath," + os.path.join(ROCM, "lib")]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("building %s failed:\n%s" % (name, r.stderr))
+        out.append(exe)
+    return out
+
+
 def build(force=True, verbose=True):
-    """Compile every .hip file and link the shared library.  Returns the library path."""
+    """Compile every .hip file and link the shared library, then the host programs.  Returns the library path."""
     if not force and up_to_date():
         return LIB
     os.makedirs(OBJ_DIR, exist_ok=True)
@@ -72,6 +96,7 @@ def build(force=True, verbose=True):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    build_host_programs()
     return LIB
 
 

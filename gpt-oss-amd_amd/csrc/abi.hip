@@ -184,6 +184,17 @@ int moe_gather_rows(const float* X, const int* idx, float* Y, int rows, int H, m
     return launch_gather_rows(X, idx, Y, rows, H, as_stream(stream));
 }
 
+int moe_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, moe_stream_t stream) {
+    if (!X || !idx || !Y) return MOE_ERR_NULL;
+    if (rows <= 0 || H <= 0 || H % 4 != 0) return MOE_ERR_SHAPE;
+    for (int r0 = 0; r0 < rows; r0 += 65535) {  // grid.y limit: slabs
+        int rc = launch_scatter_rows(Y + (size_t)r0 * H, idx + r0, X, rows - r0 < 65535 ? rows - r0 : 65535, H,
+                                     as_stream(stream));
+        if (rc) return rc;
+    }
+    return MOE_OK;
+}
+
 int moe_build_work_queue(const int* expert_offsets, int E, int* work_queue, int* work_count, moe_stream_t stream) {
     if (!expert_offsets || !work_queue || !work_count) return MOE_ERR_NULL;
     if (E <= 0) return MOE_ERR_SHAPE;

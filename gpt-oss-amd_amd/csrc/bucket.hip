@@ -120,6 +120,23 @@ int launch_gather_rows(const float* X, const int* idx, float* Y, int rows, int H
     return launch_status();
 }
 
+// X[idx[row],:] = Y[row,:]: the inverse of gather_rows (rows of a compact batch back to the table
+// rows they were gathered from; idx must not repeat).
+__global__ void scatter_rows_kernel(const float4* __restrict__ Y, const int* __restrict__ idx,
+                                    float4* __restrict__ X, int rows, int H4) {
+    const int row = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= rows || c >= H4) return;
+    X[(size_t)idx[row] * H4 + c] = Y[(size_t)row * H4 + c];
+}
+
+int launch_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, hipStream_t stream) {
+    const int H4 = H / 4;
+    hipLaunchKernelGGL(scatter_rows_kernel, dim3(ceil_div(H4, 256), rows), dim3(256), 0, stream,
+                       reinterpret_cast<const float4*>(Y), idx, reinterpret_cast<float4*>(X), rows, H4);
+    return launch_status();
+}
+
 // (expert, row_offset, row_count) triples of the non-empty experts, ascending expert id
 // (entry format of src/hip/scheduler.hip:163-166).  One wave; ballot + prefix count per 64 experts.
 __global__ __launch_bounds__(64) void work_queue_kernel(const int* __restrict__ expert_offsets, int E,

@@ -44,6 +44,7 @@ inline int tile_map_capacity(int A, int E, int tile_tokens) { return (A + tile_t
 int launch_bucket(const int* topk_i, const float* topk_v, int T, int K, int E, int* expert_offsets,
                   int* tokens_flat, float* weights_flat, int* slot_of, TileMap map, hipStream_t stream);
 int launch_gather_rows(const float* X, const int* idx, float* Y, int rows, int H, hipStream_t stream);
+int launch_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, hipStream_t stream);
 int launch_build_work_queue(const int* expert_offsets, int E, int* work_queue, int* work_count,
                             hipStream_t stream);
 

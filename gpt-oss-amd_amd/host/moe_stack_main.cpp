@@ -1,0 +1,247 @@
+// Runs the C++ host side of the library on the device: a checkpoint file goes through
+// moe_host::moe_upload_weights into stacked device tensors, then either
+//   layers  the MoE half of every layer is applied to a batch of rows with moe_host::forward_layers,
+//           the residual stream being written out after each layer, or
+//   getp    a request file goes through moe_getp::inference (the decode loop with its live-batch
+//           compaction) and the generated tokens are written in the reference's output format.
+// Usage:
+//   moe_stack_main layers <ckpt> <bin_f32|bin_bf16|safetensors:K> <x.f32> <T> <out.f32> [flags]
+//   moe_stack_main getp   <ckpt> <bin_f32|bin_bf16|safetensors:K> <in.txt> <out.txt> <steps> <batch> <vocab> <eos>
+//                         [<final_states.f32> [<step_sizes.txt>]]
+//   moe_stack_main requests <in.txt> <out.txt> <max_seq_len> [truncate]     (file formats only, no device)
+//   moe_stack_main verify <generated.txt> <ground_truth.txt>
+// MXFP4 files stay MXFP4 on the device (tiled layout); dense files are uploaded as bf16.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "moe_getp.hpp"
+
+#define CHECK_RC(expr)                                                                      \
+    do {                                                                                    \
+        const long long rc_ = (long long)(expr);                                            \
+        if (rc_ != 0) {                                                                     \
+            std::fprintf(stderr, "%s -> %lld (%s)\n", #expr, rc_, moe_error_string((int)rc_)); \
+            return 3;                                                                       \
+        }                                                                                   \
+    } while (0)
+
+template <typename T>
+static int dev_alloc(T** p, size_t count) {
+    return (int)hipMalloc((void**)p, sizeof(T) * (count ? count : 1));
+}
+
+struct Model {
+    moe_host::OssMoeTransformer tr;
+    std::vector<void*> owned;
+    ~Model() {
+        for (void* p : owned) (void)hipFree(p);
+    }
+};
+
+// kind: bin_f32 | bin_bf16 | safetensors:<experts per token> (a safetensors file does not record it; the
+// reference's exporter takes it from config.json, tools/model_export/gpt-oss-20b/export_model_bin.py:302-304)
+static int load_model(const char* path, const std::string& kind, int batch_size, Model* m) {
+    moe_ckpt* ck = nullptr;
+    int rc;
+    if (kind.rfind("safetensors", 0) == 0) {
+        moe_ckpt_config want{};  // shapes come from the file
+        want.experts_per_token = kind.size() > 12 ? std::atoi(kind.c_str() + 12) : 4;
+        want.swiglu_limit = 7.0f;
+        rc = moe_ckpt_open_safetensors(path, &want, &ck);
+    } else {
+        rc = moe_ckpt_open_bin(path, kind == "bin_bf16" ? MOE_DTYPE_BF16 : MOE_DTYPE_F32, &ck);
+    }
+    if (rc) return rc;
+    moe_host::OssMoeConfig& c = m->tr.config;
+    rc = moe_host::moe_config_from_checkpoint(ck, batch_size, &c);
+    if (rc) return rc;
+    const size_t L = c.n_layers, E = c.n_experts, H = c.hidden_dim, I = c.intermediate_dim;
+    const bool tiled = moe_ckpt_is_mxfp4(ck) != 0;
+    moe_host::OssMoeWeights& w = m->tr.weights;
+    w = moe_host::OssMoeWeights{};
+    moe_bf16_t *rms, *wr, *br, *b1, *b2, *w1 = nullptr, *w2 = nullptr;
+    uint8_t *q1 = nullptr, *s1 = nullptr, *q2 = nullptr, *s2 = nullptr;
+    if ((rc = dev_alloc(&rms, L * H)) || (rc = dev_alloc(&wr, L * E * H)) || (rc = dev_alloc(&br, L * E)) ||
+        (rc = dev_alloc(&b1, L * E * 2 * I)) || (rc = dev_alloc(&b2, L * E * H)))
+        return rc;
+    m->owned.insert(m->owned.end(), {rms, wr, br, b1, b2});
+    if (tiled) {
+        size_t bb1, sb1, bb2, sb2;
+        moe_mxfp4_tiled_bytes((int)(2 * I), (int)H, &bb1, &sb1);
+        moe_mxfp4_tiled_bytes((int)H, (int)I, &bb2, &sb2);
+        if ((rc = dev_alloc(&q1, L * E * bb1)) || (rc = dev_alloc(&s1, L * E * sb1)) || (rc = dev_alloc(&q2, L * E * bb2)) ||
+            (rc = dev_alloc(&s2, L * E * sb2)))
+            return rc;
+        m->owned.insert(m->owned.end(), {q1, s1, q2, s2});
+    } else {
+        if ((rc = dev_alloc(&w1, L * E * 2 * I * H)) || (rc = dev_alloc(&w2, L * E * H * I))) return rc;
+        m->owned.insert(m->owned.end(), {w1, w2});
+    }
+    w.rms_ffn_w = rms;
+    w.w_router = wr;
+    w.b_router = br;
+    w.b_mlp1 = b1;
+    w.b_mlp2 = b2;
+    w.w_mlp1 = w1;
+    w.w_mlp2 = w2;
+    w.w_mlp1_blocks = q1;
+    w.w_mlp1_scales = s1;
+    w.w_mlp2_blocks = q2;
+    w.w_mlp2_scales = s2;
+    const size_t staging_bytes = moe_ckpt_staging_bytes(ck);
+    uint8_t* staging;
+    if ((rc = dev_alloc(&staging, staging_bytes))) return rc;
+    rc = moe_host::moe_upload_weights(ck, c, w, staging, staging_bytes, nullptr);
+    if (!rc) rc = (int)hipDeviceSynchronize();
+    (void)hipFree(staging);
+    moe_ckpt_close(ck);
+    if (rc) return rc;
+
+    moe_host::OssMoeRunState& s = m->tr.state;
+    const size_t B = batch_size;
+    s.workspace_bytes = moe_host::moe_workspace_bytes(c);
+    uint8_t* ws;
+    if ((rc = dev_alloc(&s.x, B * H)) || (rc = dev_alloc(&s.t, B * H)) || (rc = dev_alloc(&s.e_agg, B * H)) ||
+        (rc = dev_alloc(&s.topk_v, B * c.experts_per_token)) || (rc = dev_alloc(&s.topk_i, B * c.experts_per_token)) ||
+        (rc = dev_alloc(&ws, s.workspace_bytes)))
+        return rc;
+    s.workspace = ws;
+    s.router_score = nullptr;
+    m->owned.insert(m->owned.end(), {s.x, s.t, s.e_agg, s.topk_v, s.topk_i, ws});
+    return MOE_OK;
+}
+
+static int read_floats(const char* path, std::vector<float>* out, size_t count) {
+    FILE* f = std::fopen(path, "rb");
+    if (!f) return MOE_ERR_IO;
+    out->resize(count);
+    const size_t got = std::fread(out->data(), sizeof(float), count, f);
+    std::fclose(f);
+    return got == count ? MOE_OK : MOE_ERR_IO;
+}
+
+static int run_layers(int argc, char** argv) {
+    if (argc < 7) return 2;
+    const int T = std::atoi(argv[5]);
+    Model m;
+    CHECK_RC(load_model(argv[2], argv[3], T, &m));
+    if (argc > 7) m.tr.flags = (unsigned)std::atoi(argv[7]);
+    const moe_host::OssMoeConfig& c = m.tr.config;
+    const size_t n = (size_t)T * c.hidden_dim;
+    std::vector<float> x;
+    CHECK_RC(read_floats(argv[4], &x, n));
+    CHECK_RC(hipMemcpy(m.tr.state.x, x.data(), n * sizeof(float), hipMemcpyHostToDevice));
+    FILE* out = std::fopen(argv[6], "wb");
+    if (!out) return 3;
+    std::printf("layers: %d layers, %d experts, top-%d, H=%d, I=%d, T=%d, %s experts\n", c.n_layers, c.n_experts,
+                c.experts_per_token, c.hidden_dim, c.intermediate_dim, T, m.tr.weights.w_mlp1_blocks ? "MXFP4" : "bf16");
+    // layer by layer, so that every layer's residual stream can be checked
+    for (int l = 0; l < c.n_layers; ++l) {
+        CHECK_RC(moe_host::forward_layer(&m.tr, l, T));
+        CHECK_RC(hipDeviceSynchronize());
+        CHECK_RC(hipMemcpy(x.data(), m.tr.state.x, n * sizeof(float), hipMemcpyDeviceToHost));
+        std::fwrite(x.data(), sizeof(float), n, out);
+    }
+    std::fclose(out);
+    // the whole stack again through forward() itself (every norm but the first folded into the block
+    // before it), from the same input: must equal the last dump
+    std::vector<float> x0;
+    CHECK_RC(read_floats(argv[4], &x0, n));
+    CHECK_RC(hipMemcpy(m.tr.state.x, x0.data(), n * sizeof(float), hipMemcpyHostToDevice));
+    std::vector<int> tokens(T, 0), pos(T, 0), idx(T);
+    for (int i = 0; i < T; ++i) idx[i] = i;
+    float* y = moe_host::forward(&m.tr, tokens.data(), pos.data(), T, idx.data(), T);
+    if (!y) CHECK_RC(m.tr.last_error);
+    CHECK_RC(hipDeviceSynchronize());
+    CHECK_RC(hipMemcpy(x0.data(), y, n * sizeof(float), hipMemcpyDeviceToHost));
+    if (std::memcmp(x0.data(), x.data(), n * sizeof(float)) != 0) {
+        std::fprintf(stderr, "forward() differs from the layer-by-layer result\n");
+        return 4;
+    }
+    std::printf("forward() equals the layer-by-layer result bit for bit\n");
+    return 0;
+}
+
+static int run_getp(int argc, char** argv) {
+    if (argc < 10) return 2;
+    const int steps = std::atoi(argv[6]), batch = std::atoi(argv[7]);
+    moe_getp::DecodeOptions opt;
+    opt.vocab = std::atoi(argv[8]);
+    opt.eos_token = std::atoi(argv[9]);
+    Model m;
+    CHECK_RC(load_model(argv[2], argv[3], batch, &m));
+    moe_getp::Requests reqs;
+    CHECK_RC(moe_getp::read_inputfile(argv[4], /*max_token_len=*/8, steps, &reqs, 0));
+    moe_getp::DecodeBuffers buffers;
+    std::vector<int> step_sizes;
+    std::vector<float> finals((size_t)reqs.num_reqs * m.tr.config.hidden_dim);
+    const long long n_tokens = moe_getp::inference(&m.tr, &buffers, &reqs, steps, opt, &step_sizes, finals.data());
+    if (n_tokens < 0) CHECK_RC(-n_tokens);
+    CHECK_RC(moe_getp::write_outputfile(argv[5], &reqs));
+    std::printf("getp: %d requests, batch %d, %lld tokens generated, %zu steps\n", reqs.num_reqs, batch, n_tokens,
+                step_sizes.size());
+    if (argc > 10) {
+        FILE* f = std::fopen(argv[10], "wb");
+        if (!f) return 3;
+        std::fwrite(finals.data(), sizeof(float), finals.size(), f);
+        std::fclose(f);
+    }
+    if (argc > 11) {
+        FILE* f = std::fopen(argv[11], "w");
+        if (!f) return 3;
+        for (int s : step_sizes) std::fprintf(f, "%d\n", s);
+        std::fclose(f);
+    }
+    moe_getp::free_decode_buffers(&buffers);
+    moe_getp::free_requests(&reqs);
+    return 0;
+}
+
+// requests <in.txt> <out.txt> <max_seq_len> [truncate]: reads a request file, gives request i the
+// "generated" tokens len(request i), i, i + 1, ... (len % 7 + 1 of them) and writes them out: the two
+// file formats without a device.
+static int run_requests(int argc, char** argv) {
+    if (argc < 5) return 2;
+    moe_getp::Requests reqs;
+    const int rc = moe_getp::read_inputfile(argv[2], 8, std::atoi(argv[4]), &reqs, argc > 5 ? std::atoi(argv[5]) : 0);
+    if (rc) {
+        std::printf("read_inputfile -> %d (%s)\n", rc, moe_error_string(rc));
+        return 3;
+    }
+    std::printf("num requests: %d\n", reqs.num_reqs);
+    for (int i = 0; i < reqs.num_reqs; ++i) {
+        const int len = (int)std::strlen(moe_getp::get_str_req_ptr(&reqs, i));
+        int* out = moe_getp::get_tok_gen_ptr(&reqs, i);
+        int n = len % 7 + 1;
+        if (n > reqs.max_seq_len) n = reqs.max_seq_len;
+        out[0] = len;
+        for (int j = 1; j < n; ++j) out[j] = i + j - 1;
+        out[n] = -1;
+    }
+    CHECK_RC(moe_getp::write_outputfile(argv[3], &reqs));
+    moe_getp::free_requests(&reqs);
+    return 0;
+}
+
+// verify <generated> <ground truth>: exit code 0 match, 1 mismatch, 255 unreadable
+static int run_verify(int argc, char** argv) {
+    if (argc < 4) return 2;
+    int mismatches = 0;
+    const int rc = moe_getp::verify_output(argv[2], argv[3], &mismatches, stdout);
+    std::printf("mismatches: %d\n", mismatches);
+    return rc < 0 ? 255 : rc;
+}
+
+int main(int argc, char** argv) {
+    if (argc >= 2 && std::string(argv[1]) == "requests") return run_requests(argc, argv);
+    if (argc >= 2 && std::string(argv[1]) == "verify") return run_verify(argc, argv);
+    if (argc >= 2 && std::string(argv[1]) == "layers") return run_layers(argc, argv);
+    if (argc >= 2 && std::string(argv[1]) == "getp") return run_getp(argc, argv);
+    std::fprintf(stderr, "usage: %s layers|getp|requests|verify ... (see the head of moe_stack_main.cpp)\n", argv[0]);
+    return 2;
+}

@@ -122,6 +122,12 @@ MOE_API int moe_bucket_by_expert(const int* topk_i, const float* topk_v, int B, 
  * src/forward.cpp:351-363): Y[row,:] = X[idx[row],:], fp32, H % 4 == 0. */
 MOE_API int moe_gather_rows(const float* X, const int* idx, float* Y, int rows, int H, moe_stream_t stream);
 
+/* The inverse of moe_gather_rows: X[idx[row],:] = Y[row,:] (idx without repeats).  No kernel of its
+ * own in the reference, whose per-sequence state is the KV cache, written row by row at
+ * batch_indices[row] inside split_qkv (call site src/forward.cpp:276-281); the decode loop of
+ * host/moe_getp.hpp keeps one state row per sequence instead and returns a step's rows with this. */
+MOE_API int moe_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, moe_stream_t stream);
+
 /* Replaces classify_and_build_queues (src/hip/scheduler.hip:112-184; call site
  * src/forward.cpp:373-376).  One queue of (expert, row_offset, row_count) triples for the
  * non-empty experts in ascending expert id; work_count[0] receives their number.  The
