@@ -77,6 +77,8 @@ SIGNATURES = {
     "moe_gemm_router": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
     "moe_gemm_router_static_max_bytes": (_sz, []),
     "moe_gemm_router_static": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "moe_router_two_pass_scratch_bytes": (_sz, [_i, _i, _i]),
+    "moe_router_two_pass_report": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "moe_topk": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "moe_softmax": (_i, [_vp, _i, _i, _vp]),
     "moe_bucket_by_expert": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
@@ -96,6 +98,7 @@ SIGNATURES = {
     "moe_mxfp4_tiled_to_bf16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "moe_block_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "moe_block_forward": (_i, [_c.POINTER(BlockParams), _vp]),
+    "moe_block_down_gemm": (_i, [_c.POINTER(BlockParams), _vp, _vp, _vp]),
     "moe_stage_timer_create": (_i, [_c.POINTER(_vp)]),
     "moe_stage_timer_destroy": (None, [_vp]),
     "moe_block_forward_timed": (_i, [_c.POINTER(BlockParams), _vp, _vp]),
@@ -161,6 +164,23 @@ def gemm_router_static(xout, x_batch, w, bias, N, K, M, stream=None):
     nothing is allocated (N * M limited: moe_gemm_router_static in include/moe_abi.h)."""
     _check("moe_gemm_router_static", _lib.moe_gemm_router_static(_ptr(xout), _ptr(x_batch), _ptr(w), _ptr(bias), N, K,
                                                                  M, _stream(stream)))
+
+
+def router_two_pass_report(x, w, bias, K, stream=None):
+    """The two-pass router with its intermediate results: (topk_v, topk_i, approx_scores, bound, n_candidates)."""
+    T, H = x.shape
+    E = w.shape[0]
+    dev = x.device
+    scratch = torch.empty(_lib.moe_router_two_pass_scratch_bytes(T, H, E), dtype=torch.uint8, device=dev)
+    tv = torch.empty((T, K), dtype=torch.float32, device=dev)
+    ti = torch.empty((T, K), dtype=torch.int32, device=dev)
+    approx = torch.empty((T, E), dtype=torch.float32, device=dev)
+    bound = torch.empty((T,), dtype=torch.float32, device=dev)
+    n_cand = torch.empty((T,), dtype=torch.int32, device=dev)
+    _check("moe_router_two_pass_report",
+           _lib.moe_router_two_pass_report(_ptr(x), _ptr(w), _ptr(bias), T, H, E, K, _ptr(scratch), scratch.numel(),
+                                           _ptr(tv), _ptr(ti), _ptr(approx), _ptr(bound), _ptr(n_cand), _stream(stream)))
+    return tv, ti, approx, bound, n_cand
 
 
 def topk(topk_values, topk_indices, router_scores, batch_size, num_experts, experts_per_token, stream=None):
@@ -322,7 +342,7 @@ class MoeBlock:
 
     def params(self, t, e_agg, topk_i, topk_v, router_score=None, residual_x=None, flags=0, next_norm_weight=None,
                next_norm_out=None):
-        T = t.shape[0]
+        T = t.shape[0] if t is not None else topk_i.shape[0]
         p = BlockParams()
         p.struct_bytes = ctypes.sizeof(BlockParams)
         p.n_tokens, p.hidden_dim, p.intermediate_dim = T, self.H, self.I
@@ -351,6 +371,17 @@ class MoeBlock:
         p = self.params(t, e_agg, topk_i, topk_v, router_score, residual_x, flags, next_norm_weight, next_norm_out)
         _check("moe_block_forward", _lib.moe_block_forward(ctypes.byref(p), _stream(stream)))
         return e_agg, topk_i, topk_v
+
+    def down_gemm(self, topk_i, h_by_assignment, flags=0, stream=None):
+        """The block's down-projection GEMM alone: bf16 rows [T*K, I] by assignment -> fp32 rows [T*K, H]."""
+        T = topk_i.shape[0]
+        y = torch.empty((T * self.K, self.H), dtype=torch.float32, device=topk_i.device)
+        tv = torch.ones((T, self.K), dtype=torch.float32, device=topk_i.device)
+        p = self.params(None, None, topk_i, tv, flags=flags)
+        p.n_tokens = T
+        _check("moe_block_down_gemm", _lib.moe_block_down_gemm(ctypes.byref(p), _ptr(h_by_assignment), _ptr(y),
+                                                               _stream(stream)))
+        return y
 
     def launch(self, p, stream):
         """Re-issue a prepared parameter block (benchmark loop: no Python-side tensor work)."""

@@ -5,6 +5,7 @@
 #include "kernels.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstddef>
 #include <cstring>
 #include <new>
@@ -139,6 +140,25 @@ int moe_gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, cons
     int rc = launch_router_partial(x_batch, w, partial, nullptr, N, K, M, S, as_stream(stream));
     if (rc) return rc;
     return launch_router_finalize(partial, S, nullptr, bias, xout, nullptr, nullptr, N, M, 0, 0, 0, as_stream(stream));
+}
+
+size_t moe_router_two_pass_scratch_bytes(int N, int K, int M) {
+    if (N <= 0 || K <= 0 || M <= 0 || K % 32 != 0) return 0;
+    return router_screen_bytes(N, M, K);
+}
+
+int moe_router_two_pass_report(const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias, int N, int K, int M,
+                               int experts_per_token, void* scratch, size_t scratch_bytes, float* topk_values,
+                               int* topk_indices, float* approx_scores, float* bound, int* n_candidates,
+                               moe_stream_t stream) {
+    if (!x_batch || !w || !bias || !topk_values || !topk_indices) return MOE_ERR_NULL;
+    if (N <= 0 || K <= 0 || M <= 0 || K % 32 != 0 || experts_per_token <= 0 || experts_per_token > M)
+        return MOE_ERR_SHAPE;
+    if (M > 1024 || experts_per_token > 8) return MOE_ERR_LIMIT;
+    if (((uintptr_t)x_batch | (uintptr_t)w) & 15u) return MOE_ERR_ALIGN;
+    if (!scratch || ((uintptr_t)scratch & 15u) || scratch_bytes < router_screen_bytes(N, M, K)) return MOE_ERR_WORKSPACE;
+    return launch_router_two_pass(x_batch, w, bias, scratch, nullptr, topk_values, topk_indices, N, K, M,
+                                  experts_per_token, 1, as_stream(stream), nullptr, approx_scores, bound, n_candidates);
 }
 
 int moe_topk(float* topk_values, int* topk_indices, const float* router_scores, int batch_size, int num_experts,
@@ -358,6 +378,106 @@ struct moe_stage_timer {
     hipEvent_t ev[MOE_N_STAGES + 1];
 };
 
+// Compute units of the current device, asked once per device (the kernel choices below count rounds
+// of blocks over them).
+static int device_cu_count() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+// Launch parameters of the two expert GEMMs of one block.
+struct ExpertPlan {
+    const moe_block_params* p;
+    ExpertGemmArgs g{};
+    bool prefill, direct;
+    int est_tiles, n_cus;
+
+    ExpertPlan(const moe_block_params* p_, const BlockWorkspace& ws, bool prefill_, bool direct_, int tile_tokens,
+               int max_tiles)
+        : p(p_), prefill(prefill_), direct(direct_) {
+        const int T = p->n_tokens, E = p->n_experts, K = p->experts_per_token;
+        g.tokens_flat = ws.tokens_flat;
+        g.tile_expert = ws.tile_expert;
+        g.tile_row0 = ws.tile_row0;
+        g.tile_rows = ws.tile_rows;
+        g.n_tiles = ws.n_tiles;
+        g.max_tiles = max_tiles;
+        g.alpha = p->alpha;
+        g.limit = p->swiglu_limit;
+        g.format = p->weight_format;
+        if (direct) {
+            g.topk_i = p->topk_i;
+            g.n_assign = T * K;
+            g.assign_div = K;
+            g.n_experts = E;
+        }
+        est_tiles = direct ? E : std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
+        n_cus = device_cu_count();
+    }
+    // Decode-sized buckets (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of
+    // 32 rows each.  Blocks run in rounds of one per CU, so the cheaper choice is the one with the
+    // smaller rounds x rows-per-block product; more rows per block also re-read the activations less.
+    int pick_kernel(int rows) const {
+        if (prefill) return 16;
+        const int cost10 = ceil_div(ceil_div(rows / 32, 10) * est_tiles, n_cus) * 10;
+        const int cost12 = ceil_div(ceil_div(rows / 32, 12) * est_tiles, n_cus) * 12;
+        return cost12 <= cost10 ? 1 : 0;
+    }
+    // one row block more than necessary when that makes the block count a whole number of rounds
+    int pick_row_blocks(int rows, int kernel) const {
+        if (prefill) return 0;
+        const int n = ceil_div(rows / 32, kernel == 1 ? 12 : 10);
+        return ((n * est_tiles) % n_cus != 0 && ((n + 1) * est_tiles) % n_cus == 0) ? n + 1 : n;
+    }
+    void set_weights(ExpertGemmArgs& a, const void* w, const void* scales, int rows, int Kdim) const {
+        a.w = w;
+        a.w_scales = static_cast<const uint8_t*>(scales);
+        a.rows = rows;
+        a.K = Kdim;
+        a.bias_expert_stride = rows;
+        a.waves_per_block = pick_kernel(rows);
+        a.row_blocks = pick_row_blocks(rows, a.waves_per_block);
+        if (p->weight_format == MOE_WEIGHTS_BF16) {
+            a.w_expert_stride = (long long)rows * Kdim;
+        } else {
+            size_t bb, sb;
+            mxfp4_tiled_bytes(rows, Kdim, &bb, &sb);
+            a.w_expert_stride = (long long)bb;
+            a.s_expert_stride = (long long)sb;
+        }
+    }
+    // act: bf16 [T, H] rows gathered by token; out: bf16 SwiGLU rows [A, I]
+    ExpertGemmArgs gate_up(const uint16_t* act, uint16_t* out) const {
+        ExpertGemmArgs a = g;
+        set_weights(a, p->w_mlp1, p->w_mlp1_scales, 2 * p->intermediate_dim, p->hidden_dim);
+        a.bias = p->b_mlp1;
+        a.act = act;
+        a.gather = 1;
+        a.out = out;
+        return a;
+    }
+    // act: bf16 [A, I] rows (by slot, or by assignment when bucketing is done in the kernel); out: fp32 [A, H]
+    ExpertGemmArgs down(const uint16_t* act, float* out) const {
+        ExpertGemmArgs a = g;
+        set_weights(a, p->w_mlp2, p->w_mlp2_scales, p->hidden_dim, p->intermediate_dim);
+        a.bias = p->b_mlp2;
+        a.act = act;
+        a.gather = 0;
+        a.out = out;
+        // measured: the down GEMM gains 4-10 % from keeping a token block on one XCD (its input rows were
+        // written by the gate/up launch just before), the gate/up GEMM loses up to 2 %
+        a.xcd_tiles = 1;
+        return a;
+    }
+};
+
 static int block_forward_impl(const moe_block_params* caller, moe_stream_t stream_, moe_stage_timer* timer) {
     if (!caller) return MOE_ERR_NULL;
     // the struct as it was before next_norm_weight / next_norm_out were appended is still accepted
@@ -434,90 +554,14 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     if ((rc = mark())) return rc;
 
     // 3. gate/up GEMM + SwiGLU  (src/forward.cpp:474-479; src/run.cpp:657-689)
-    ExpertGemmArgs g{};
-    g.tokens_flat = ws.tokens_flat;
-    g.tile_expert = ws.tile_expert;
-    g.tile_row0 = ws.tile_row0;
-    g.tile_rows = ws.tile_rows;
-    g.n_tiles = ws.n_tiles;
-    g.max_tiles = max_tiles;
-    g.alpha = p->alpha;
-    g.limit = p->swiglu_limit;
-    g.format = fmt;
-    if (direct) {
-        g.topk_i = p->topk_i;
-        g.n_assign = T * K;
-        g.assign_div = K;
-        g.n_experts = E;
-    }
-
-    // Decode-sized buckets (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of
-    // 32 rows each.  Blocks run in rounds of one per CU, so the cheaper choice is the one with the
-    // smaller rounds x rows-per-block product; more rows per block also re-read the activations less.
-    const int est_tiles = direct ? E : std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
-    const int kCUs = 256;  // MI355X
-    auto pick_consumers = [&](int rows) {
-        const int cost10 = ceil_div(ceil_div(rows / 32, 10) * est_tiles, kCUs) * 10;
-        const int cost12 = ceil_div(ceil_div(rows / 32, 12) * est_tiles, kCUs) * 12;
-        return cost12 <= cost10 ? 1 : 0;
-    };
-    // one row block more than necessary when that makes the block count a whole number of rounds
-    auto pick_row_blocks = [&](int rows, int kernel) {
-        const int p = ceil_div(rows / 32, kernel == 1 ? 12 : 10);
-        return ((p * est_tiles) % kCUs != 0 && ((p + 1) * est_tiles) % kCUs == 0) ? p + 1 : p;
-    };
-    auto pick_kernel = [&](int rows) {
-        return prefill ? 16 : pick_consumers(rows);
-    };
-
-    ExpertGemmArgs a1 = g;
-    a1.w = p->w_mlp1;
-    a1.w_scales = static_cast<const uint8_t*>(p->w_mlp1_scales);
-    a1.bias = p->b_mlp1;
-    a1.act = ws.t_bf16;
-    a1.gather = 1;
-    a1.out = ws.h_by_slot;
-    a1.rows = 2 * I;
-    a1.K = H;
-    a1.bias_expert_stride = 2LL * I;
-    a1.waves_per_block = pick_kernel(2 * I);
-    a1.row_blocks = prefill ? 0 : pick_row_blocks(2 * I, a1.waves_per_block);
-    if (fmt == MOE_WEIGHTS_BF16) {
-        a1.w_expert_stride = 2LL * I * H;
-    } else {
-        size_t bb, sb;
-        mxfp4_tiled_bytes(2 * I, H, &bb, &sb);
-        a1.w_expert_stride = (long long)bb;
-        a1.s_expert_stride = (long long)sb;
-    }
+    const ExpertPlan plan(p, ws, prefill, direct, tile_tokens, max_tiles);
+    const ExpertGemmArgs a1 = plan.gate_up(ws.t_bf16, ws.h_by_slot);
     rc = launch_expert_stream(a1, 0, stream);
     if (rc) return rc;
     if ((rc = mark())) return rc;
 
     // 4. down GEMM  (src/forward.cpp:481-487; src/run.cpp:691-700)
-    ExpertGemmArgs a2 = g;
-    a2.w = p->w_mlp2;
-    a2.w_scales = static_cast<const uint8_t*>(p->w_mlp2_scales);
-    a2.bias = p->b_mlp2;
-    a2.act = ws.h_by_slot;
-    a2.gather = 0;
-    a2.out = ws.y_by_slot;
-    a2.rows = H;
-    a2.K = I;
-    a2.bias_expert_stride = H;
-    a2.waves_per_block = pick_kernel(H);
-    a2.row_blocks = prefill ? 0 : pick_row_blocks(H, a2.waves_per_block);
-    // measured: the down GEMM gains 4-10 % from keeping a token block on one XCD (its input rows were
-    // written by the gate/up launch just before), the gate/up GEMM loses up to 2 %
-    a2.xcd_tiles = 1;
-    if (fmt == MOE_WEIGHTS_BF16) {
-        a2.w_expert_stride = (long long)H * I;
-    } else {
-        size_t bb, sb;
-        mxfp4_tiled_bytes(H, I, &bb, &sb);
-        a2.w_expert_stride = (long long)bb;
-        a2.s_expert_stride = (long long)sb;
-    }
+    const ExpertGemmArgs a2 = plan.down(ws.h_by_slot, ws.y_by_slot);
     rc = launch_expert_stream(a2, 1, stream);
     if (rc) return rc;
     if ((rc = mark())) return rc;
@@ -539,6 +583,44 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
 }
 
 int moe_block_forward(const moe_block_params* p, moe_stream_t stream) { return block_forward_impl(p, stream, nullptr); }
+
+int moe_block_down_gemm(const moe_block_params* caller, const moe_bf16_t* h_by_assignment, float* y_by_assignment,
+                        moe_stream_t stream_) {
+    if (!caller || !h_by_assignment || !y_by_assignment) return MOE_ERR_NULL;
+    if (caller->struct_bytes != sizeof(moe_block_params)) return MOE_ERR_FORMAT;
+    const moe_block_params* p = caller;
+    const int T = p->n_tokens, H = p->hidden_dim, I = p->intermediate_dim, E = p->n_experts,
+              K = p->experts_per_token;
+    int rc = check_dims(T, H, I, E, K);
+    if (rc) return rc;
+    if (!p->w_mlp2 || !p->b_mlp2 || !p->topk_i || !p->topk_v) return MOE_ERR_NULL;
+    const int fmt = p->weight_format;
+    if (fmt != MOE_WEIGHTS_BF16 && fmt != MOE_WEIGHTS_MXFP4_TILED) return MOE_ERR_FORMAT;
+    if (fmt == MOE_WEIGHTS_MXFP4_TILED && !p->w_mlp2_scales) return MOE_ERR_NULL;
+    if (((uintptr_t)h_by_assignment | (uintptr_t)y_by_assignment | (uintptr_t)p->w_mlp2) & 15u) return MOE_ERR_ALIGN;
+    if (!p->workspace || ((uintptr_t)p->workspace & (kAlign - 1))) return MOE_ERR_WORKSPACE;
+    BlockWorkspace ws(p->workspace, T, H, I, E, K);
+    if (p->workspace_bytes < ws.bytes) return MOE_ERR_WORKSPACE;
+    hipStream_t stream = as_stream(stream_);
+    const bool prefill = use_prefill_kernels(T, K, E, fmt, p->flags);
+    const bool direct = use_direct_bucketing(T, K, E, prefill, p->flags);
+    const int tile_tokens = prefill ? kPrefillTileTokens : kStreamTileTokens;
+    const int max_tiles = tile_map_capacity(T * K, E, tile_tokens);
+    const ExpertPlan plan(p, ws, prefill, direct, tile_tokens, max_tiles);
+    if (direct) return launch_expert_stream(plan.down(h_by_assignment, y_by_assignment), 1, stream);
+    // rows by slot: bucket, bring the caller's rows into slot order, multiply, bring the result back
+    TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles};
+    rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat, ws.slot_of,
+                       map, stream);
+    if (rc) return rc;
+    // a bf16 row of I values is moved as I/2 floats
+    rc = launch_scatter_rows(reinterpret_cast<const float*>(h_by_assignment), ws.slot_of,
+                             reinterpret_cast<float*>(ws.h_by_slot), T * K, I / 2, stream);
+    if (rc) return rc;
+    rc = launch_expert_stream(plan.down(ws.h_by_slot, ws.y_by_slot), 1, stream);
+    if (rc) return rc;
+    return launch_gather_rows(ws.y_by_slot, ws.slot_of, y_by_assignment, T * K, H, stream);
+}
 
 int moe_block_forward_timed(const moe_block_params* p, moe_stream_t stream, moe_stage_timer* timer) {
     if (!timer) return MOE_ERR_NULL;

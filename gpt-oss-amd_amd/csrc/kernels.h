@@ -26,7 +26,8 @@ bool router_two_pass(int T, int E, int H);
 size_t router_screen_bytes(int T, int E, int H);
 int launch_router_two_pass(const float* x, const uint16_t* w, const uint16_t* bias, void* scratch, uint16_t* x_bf16,
                            float* topk_v, int* topk_i, int T, int H, int E, int K, int do_softmax,
-                           hipStream_t stream, hipEvent_t between);
+                           hipStream_t stream, hipEvent_t between, float* approx_out = nullptr,
+                           float* delta_out = nullptr, int* n_cand_out = nullptr);
 
 // ---- bucket.hip -------------------------------------------------------------------------------
 // Token-block map consumed by the expert kernels: tile i covers rows

@@ -661,7 +661,10 @@ __global__ __launch_bounds__(256, 4) void router_refine_kernel(const float* __re
                                                             const uint16_t* __restrict__ w,
                                                             const uint16_t* __restrict__ bias, float err_coeff,
                                                             float* __restrict__ topk_v, int* __restrict__ topk_i,
-                                                            int T, int H, int E, int K, int do_softmax) {
+                                                            int T, int H, int E, int K, int do_softmax,
+                                                            float* __restrict__ approx_out,
+                                                            float* __restrict__ delta_out,
+                                                            int* __restrict__ n_cand_out) {
     extern __shared__ float sc[];
     __shared__ float w2_of_wave[4];
     const int lane = threadIdx.x & 63;
@@ -723,6 +726,7 @@ __global__ __launch_bounds__(256, 4) void router_refine_kernel(const float* __re
         approx[e] = v;
         exact[e] = -INFINITY;
         amax = fmaxf(amax, fabsf(v));
+        if (approx_out) approx_out[(size_t)t * E + e] = v;  // what the screening decides on, for whoever checks the bound
     }
     amax = wave_max_nonneg(amax);
     // upper bound of |approx - exact| for every expert of this token; the 1.001 factors cover the
@@ -747,6 +751,10 @@ __global__ __launch_bounds__(256, 4) void router_refine_kernel(const float* __re
     if (n_cand < K) {  // not-a-number scores: no screening, every expert is scored exactly
         for (int e = lane; e < E; e += 64) cand[e] = e;
         n_cand = E;
+    }
+    if (lane == 0) {
+        if (delta_out) delta_out[t] = delta;
+        if (n_cand_out) n_cand_out[t] = n_cand;
     }
     __builtin_amdgcn_wave_barrier();
 
@@ -859,7 +867,8 @@ size_t router_screen_bytes(int T, int E, int H) {
 
 int launch_router_two_pass(const float* x, const uint16_t* w, const uint16_t* bias, void* scratch, uint16_t* x_bf16,
                            float* topk_v, int* topk_i, int T, int H, int E, int K, int do_softmax,
-                           hipStream_t stream, hipEvent_t between) {
+                           hipStream_t stream, hipEvent_t between, float* approx_out, float* delta_out,
+                           int* n_cand_out) {
     int seg_len, S;
     screen_plan(T, E, H, &seg_len, &S);
     float* partial = static_cast<float*>(scratch);
@@ -887,7 +896,7 @@ int launch_router_two_pass(const float* x, const uint16_t* w, const uint16_t* bi
     const float err_coeff = ((float)(33 + 2 * (seg_len / 32)) * 0x1p-23f + 0x1p-16f + 8 * 0x1p-24f) * 1.01f;
     hipLaunchKernelGGL(router_refine_kernel, dim3(ceil_div(T, 4)), dim3(256),
                        (size_t)4 * 3 * E * sizeof(float), stream, partial, S, wn2, xn2, x, w, bias, err_coeff, topk_v,
-                       topk_i, T, H, E, K, do_softmax);
+                       topk_i, T, H, E, K, do_softmax, approx_out, delta_out, n_cand_out);
     return launch_status();
 }
 

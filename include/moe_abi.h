@@ -91,6 +91,22 @@ MOE_API size_t moe_gemm_router_static_max_bytes(void);
 MOE_API int moe_gemm_router_static(float* xout, const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias,
                            int N, int K, int M, moe_stream_t stream);
 
+/* The two-pass router that moe_block_forward uses for large batches, on its own and with its
+ * intermediate results (no counterpart in the reference; same top-k and softmax weights as
+ * moe_gemm_router + moe_topk + moe_softmax).  Pass 1 scores every expert approximately on the
+ * matrix cores; pass 2 bounds the error of those scores per token, recomputes exactly (the
+ * arithmetic of src/run.cpp:341-354) every expert whose approximate score is within twice the bound
+ * of the K-th best, and selects among the exact scores.  Outputs besides topk_values / topk_indices
+ * [N, experts_per_token], each optional: approx_scores [N, M] (pass 1, bias included), bound [N]
+ * (the error bound pass 2 used), n_candidates [N] (experts rescored exactly).  A caller can thus
+ * check the bound against exact scores of its own.  K % 32 == 0; scratch of
+ * moe_router_two_pass_scratch_bytes(N, K, M) bytes, 16-byte aligned. */
+MOE_API size_t moe_router_two_pass_scratch_bytes(int N, int K, int M);
+MOE_API int moe_router_two_pass_report(const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias, int N,
+                               int K, int M, int experts_per_token, void* scratch, size_t scratch_bytes,
+                               float* topk_values, int* topk_indices, float* approx_scores, float* bound,
+                               int* n_candidates, moe_stream_t stream);
+
 /* Replaces topk (src/hip/topk.hip:59-72; call site src/forward.cpp:325).  Per token the
  * experts_per_token largest scores in descending order with their indices; equal scores keep
  * the lower expert index first (the order the reference's CPU qsort yields, src/run.cpp:373-404).
@@ -271,6 +287,17 @@ enum {
 MOE_API size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int intermediate_dim, int n_experts,
                                  int experts_per_token);
 MOE_API int moe_block_forward(const moe_block_params* params, moe_stream_t stream);
+
+/* The down-projection GEMM of moe_block_forward on its own, on rows the caller provides (the
+ * kernels that stand in for moe_mlp2_scatter_mfma_kernel, src/hip/moe.hip:261-512, without the
+ * scatter): for every assignment (t, k), row t * K + k,
+ *   y_by_assignment[t*K+k, :] = W2_e h_by_assignment[t*K+k, :] + b2_e,   e = params->topk_i[t, k].
+ * params as for moe_block_forward with topk_i [B,K] as INPUT (distinct expert ids per token) and
+ * t, w_router, b_router, w_mlp1, b_mlp1, e_agg unused; the same size rules and flags choose the
+ * kernels, so a caller can put known rows (say unit vectors) through exactly the code the block
+ * runs.  h_by_assignment: bf16 [B*K, I]; y_by_assignment: fp32 [B*K, H]; both 16-byte aligned. */
+MOE_API int moe_block_down_gemm(const moe_block_params* params, const moe_bf16_t* h_by_assignment,
+                        float* y_by_assignment, moe_stream_t stream);
 
 /* Per-stage timing of moe_block_forward with HIP events on the caller's stream.  Stands in for
  * the reference's batch timing hooks, which its runtime calls but defines nowhere
