@@ -98,6 +98,8 @@ SIGNATURES = {
     "moe_mxfp4_tiled_to_bf16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "moe_block_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "moe_block_forward": (_i, [_c.POINTER(BlockParams), _vp]),
+    "moe_block_describe": (_i, [_c.POINTER(BlockParams), _c.c_char_p, _sz]),
+    "moe_synth_normal_table": (None, [_vp]),
     "moe_block_down_gemm": (_i, [_c.POINTER(BlockParams), _vp, _vp, _vp]),
     "moe_stage_timer_create": (_i, [_c.POINTER(_vp)]),
     "moe_stage_timer_destroy": (None, [_vp]),
@@ -383,6 +385,12 @@ class MoeBlock:
                                                                _stream(stream)))
         return y
 
+    def describe(self, p):
+        """Which kernels moe_block_forward launches for parameter block p: dict of the 'key=value' parts."""
+        buf = ctypes.create_string_buffer(1024)
+        _check("moe_block_describe", _lib.moe_block_describe(ctypes.byref(p), buf, len(buf)))
+        return dict(part.split("=", 1) for part in buf.value.decode().split("; "))
+
     def launch(self, p, stream):
         """Re-issue a prepared parameter block (benchmark loop: no Python-side tensor work)."""
         rc = _lib.moe_block_forward(ctypes.byref(p), stream)
@@ -418,6 +426,15 @@ class StageTimer:
 
 
 # ---- synthetic workloads (include/moe_synth.h) --------------------------------------------------
+def normal_table():
+    """The generator's table of N(0,1) quantiles (numpy float32 [65536]), built by the library."""
+    import numpy as np
+    table = np.empty(1 << 16, dtype=np.float32)
+    _lib.moe_synth_normal_table(table.ctypes.data)
+    return table
+
+
+
 def synth_normal_f32(dst, table_d, scale, seed, tensor_id, stream=None):
     _check("moe_synth_normal_f32", _lib.moe_synth_normal_f32(_ptr(dst), dst.numel(), _ptr(table_d), scale, seed,
                                                              tensor_id, _stream(stream)))

@@ -1,12 +1,14 @@
 // extern "C" entry points of libmoe_gfx950.so (declared in include/moe_abi.h): argument checks,
 // workspace carving and launch sequencing.  No entry allocates, synchronises or exits.
 #include "../../include/moe_checkpoint.h"
+#include "../../include/moe_synth.h"
 #include "common.h"
 #include "kernels.h"
 
 #include <algorithm>
 #include <atomic>
 #include <cstddef>
+#include <cstdio>
 #include <cstring>
 #include <new>
 
@@ -583,6 +585,49 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
 }
 
 int moe_block_forward(const moe_block_params* p, moe_stream_t stream) { return block_forward_impl(p, stream, nullptr); }
+
+int moe_block_describe(const moe_block_params* p, char* text, size_t text_bytes) {
+    if (!p || !text) return MOE_ERR_NULL;
+    if (text_bytes < 64) return MOE_ERR_LIMIT;
+    if (p->struct_bytes != sizeof(moe_block_params) && p->struct_bytes != offsetof(moe_block_params, next_norm_weight))
+        return MOE_ERR_FORMAT;
+    const int T = p->n_tokens, H = p->hidden_dim, I = p->intermediate_dim, E = p->n_experts,
+              K = p->experts_per_token;
+    int rc = check_dims(T, H, I, E, K);
+    if (rc) return rc;
+    const int fmt = p->weight_format;
+    if (fmt != MOE_WEIGHTS_BF16 && fmt != MOE_WEIGHTS_MXFP4_TILED) return MOE_ERR_FORMAT;
+    // the same decisions, in the same order, as block_forward_impl
+    const bool strict = (p->flags & MOE_FLAG_ROUTER_STRICT_ORDER) != 0;
+    const char* router = (!strict && !p->router_score && router_two_pass(T, E, H))
+                             ? "router_screen_kernel + router_refine_kernel"
+                             : (!strict && router_fused_fits(H)) ? "router_fused_kernel"
+                                                                 : "router_partial_kernel + router_finalize_kernel";
+    const bool prefill = use_prefill_kernels(T, K, E, fmt, p->flags);
+    const bool direct = use_direct_bucketing(T, K, E, prefill, p->flags);
+    const int tile_tokens = prefill ? kPrefillTileTokens : kStreamTileTokens;
+    BlockWorkspace ws(nullptr, T, H, I, E, K);
+    const ExpertPlan plan(p, ws, prefill, direct, tile_tokens, tile_map_capacity(T * K, E, tile_tokens));
+    auto gemm_name = [&](int rows, int epi, char* out, size_t n) {
+        const int kernel = plan.pick_kernel(rows);
+        if (prefill) snprintf(out, n, "expert_prefill_kernel<%d, %d, 4>", fmt, epi);
+        else snprintf(out, n, "%s<%d, %d, %d, 2>", direct ? "expert_stream_direct_kernel" : "expert_stream_ws_kernel", fmt,
+                      epi, kernel == 1 ? 12 : 10);
+    };
+    char g1[96], g2[96];
+    gemm_name(2 * I, 0, g1, sizeof(g1));
+    gemm_name(H, 1, g2, sizeof(g2));
+    const int n = snprintf(text, text_bytes, "router=%s; bucketing=%s; gate_up=%s; down=%s; combine=%s; compute_units=%d",
+                           router, direct ? "in the expert kernels" : "bucket_kernel", g1, g2,
+                           p->next_norm_out ? "combine_norm_kernel" : "combine_kernel", plan.n_cus);
+    return (n < 0 || (size_t)n >= text_bytes) ? MOE_ERR_LIMIT : MOE_OK;
+}
+
+void moe_synth_normal_table(float* h_table) {
+#if !defined(__HIP_DEVICE_COMPILE__)  // the builder exists in the host pass only (libm)
+    if (h_table) moe_synth_build_normal_table(h_table);
+#endif
+}
 
 int moe_block_down_gemm(const moe_block_params* caller, const moe_bf16_t* h_by_assignment, float* y_by_assignment,
                         moe_stream_t stream_) {

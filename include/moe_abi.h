@@ -288,6 +288,13 @@ MOE_API size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int inter
                                  int experts_per_token);
 MOE_API int moe_block_forward(const moe_block_params* params, moe_stream_t stream);
 
+/* Which kernels moe_block_forward would launch for these parameters (shapes, format, flags and
+ * whether router_score / next_norm_out are set; pointers are not dereferenced and may be NULL), as
+ * one line of text: "router=...; bucketing=...; gate_up=<kernel name as a profiler shows it>;
+ * down=...; combine=...; compute_units=N".  For benchmarks and profile summaries that have to name
+ * the kernel they measured.  text_bytes >= 64; MOE_ERR_LIMIT if the line does not fit. */
+MOE_API int moe_block_describe(const moe_block_params* params, char* text, size_t text_bytes);
+
 /* The down-projection GEMM of moe_block_forward on its own, on rows the caller provides (the
  * kernels that stand in for moe_mlp2_scatter_mfma_kernel, src/hip/moe.hip:261-512, without the
  * scatter): for every assignment (t, k), row t * K + k,
@@ -317,6 +324,9 @@ MOE_API int moe_stage_timer_read(moe_stage_timer* timer, float* stage_ms);
  * Synthetic workload generator (include/moe_synth.h), device side: fills device buffers with
  * the same values the host generator produces for (seed, tensor_id, index).
  * ---------------------------------------------------------------------------------------- */
+/* Host side: the 65536-entry table of N(0,1) quantiles the normal generators index
+ * (moe_synth_build_normal_table of include/moe_synth.h); h_table has room for 65536 floats. */
+MOE_API void moe_synth_normal_table(float* h_table);
 MOE_API int moe_synth_normal_f32(float* dst, long long n, const float* table_d, float scale, unsigned seed,
                          unsigned tensor_id, moe_stream_t stream);
 MOE_API int moe_synth_normal_bf16(moe_bf16_t* dst, long long n, const float* table_d, float scale,
