@@ -438,14 +438,40 @@ struct ExpertPlan {
         const int n = ceil_div(rows / 32, kernel == 1 ? 12 : 10);
         return ((n * est_tiles) % n_cus != 0 && ((n + 1) * est_tiles) % n_cus == 0) ? n + 1 : n;
     }
+    // MXFP4 with the bucketing inside the kernel: a block may cover up to two passes of CONS row units
+    // (the second pass starts with its weights already in flight), so fewer, longer blocks pay fewer
+    // pipeline fills.  Time of a round of blocks ~ one fill + passes x stages x consumers / 12; all
+    // (consumers, row blocks) choices that keep every compute unit busy are priced.
+    void pick_two_pass(int rows, int* kernel, int* row_blocks) const {
+        const int units = rows / 32;
+        double best = 1e30;
+        for (int k = 0; k < 2; ++k) {
+            const int cons = k == 1 ? 12 : 10;
+            for (int n = ceil_div(units, 2 * cons); n <= ceil_div(units, cons); ++n) {
+                const int per_block = ceil_div(units, n);
+                const int passes = ceil_div(per_block, cons);
+                const int rounds = ceil_div(n * est_tiles, n_cus);
+                const double cost = rounds * (6.0 + passes * 25.0 * cons / 12.0);
+                if (cost < best - 1e-9) {
+                    best = cost;
+                    *kernel = k;
+                    *row_blocks = n;
+                }
+            }
+        }
+    }
     void set_weights(ExpertGemmArgs& a, const void* w, const void* scales, int rows, int Kdim) const {
         a.w = w;
         a.w_scales = static_cast<const uint8_t*>(scales);
         a.rows = rows;
         a.K = Kdim;
         a.bias_expert_stride = rows;
-        a.waves_per_block = pick_kernel(rows);
-        a.row_blocks = pick_row_blocks(rows, a.waves_per_block);
+        if (direct && p->weight_format == MOE_WEIGHTS_MXFP4_TILED) {
+            pick_two_pass(rows, &a.waves_per_block, &a.row_blocks);
+        } else {
+            a.waves_per_block = pick_kernel(rows);
+            a.row_blocks = pick_row_blocks(rows, a.waves_per_block);
+        }
         if (p->weight_format == MOE_WEIGHTS_BF16) {
             a.w_expert_stride = (long long)rows * Kdim;
         } else {
@@ -609,7 +635,8 @@ int moe_block_describe(const moe_block_params* p, char* text, size_t text_bytes)
     BlockWorkspace ws(nullptr, T, H, I, E, K);
     const ExpertPlan plan(p, ws, prefill, direct, tile_tokens, tile_map_capacity(T * K, E, tile_tokens));
     auto gemm_name = [&](int rows, int epi, char* out, size_t n) {
-        const int kernel = plan.pick_kernel(rows);
+        int kernel = plan.pick_kernel(rows), unused = 0;
+        if (direct && fmt == MOE_WEIGHTS_MXFP4_TILED) plan.pick_two_pass(rows, &kernel, &unused);
         if (prefill) snprintf(out, n, "expert_prefill_kernel<%d, %d, 4>", fmt, epi);
         else snprintf(out, n, "%s<%d, %d, %d, 2>", direct ? "expert_stream_direct_kernel" : "expert_stream_ws_kernel", fmt,
                       epi, kernel == 1 ? 12 : 10);

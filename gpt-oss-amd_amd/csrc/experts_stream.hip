@@ -394,8 +394,10 @@ MOE_DEVICE int ws_chunk(int j, int g) {  // chunk holding the operand of MFMA st
 }
 
 // act_row(i): row of a.act that holds bucket row i of the token block (i < nrows).
+// The stages of the bucket's rows are streamed `passes` times over (once per pass of the consumers
+// over their row units), without a break in between.
 template <int FMT, int NT, int PROD, class RowFn>
-MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row, int nrows, int p) {
+MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row, int nrows, int p, int passes) {
     constexpr int BP = 4 / PROD;  // four-row blocks of a token tile moved by this wave
     constexpr int Q = BP * NT;    // direct-to-LDS loads per stage issued by this wave
     const int lane = threadIdx.x & 63;
@@ -421,11 +423,12 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row
             row[t][ii] = reinterpret_cast<const uint8_t*>(a.act + (size_t)act_row(idx) * K);
         }
     }
-    auto issue = [&](int s) {
-        uint8_t* slot = lds + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes;
+    // stage st of the rows into ring slot gs % 4 (gs counts stages over all passes)
+    auto issue = [&](int gs, int st) {
+        uint8_t* slot = lds + (size_t)(gs & (kWsRing - 1)) * kLdsStageBytes;
 #pragma unroll
         for (int ii = 0; ii < BP; ++ii) {
-            const int k = s * kStageElems + 8 * chunk[ii];
+            const int k = st * kStageElems + 8 * chunk[ii];
             const size_t off = (k < K) ? (size_t)k * 2 : 0;  // a position past the row re-reads its start
 #pragma unroll
             for (int t = 0; t < NT; ++t)
@@ -443,13 +446,18 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row
     // every outstanding direct-to-LDS load (vmcnt(0)) in front of each barrier, i.e. also for the
     // stages issued just now, and the ring would hide nothing.  The explicit wait above each barrier
     // is the guarantee the consumers need: the stage they read next has been written to LDS.
-    issue(0);
-    issue(1);
-    issue(2);
+    int st = 0;  // stage (inside a pass) issued next
+    auto next_stage = [&]() { st = (st + 1 == n_stages) ? 0 : st + 1; };
+    for (int gs = 0; gs < 3; ++gs) {
+        issue(gs, st);
+        next_stage();
+    }
     wait_two_stages();  // stage 0 has landed
     __builtin_amdgcn_s_barrier();
-    for (int i = 0; i < n_stages; ++i) {
-        issue(i + 3);  // past the last stage: a re-read nobody consumes
+    const int total = passes * n_stages;
+    for (int i = 0; i < total; ++i) {
+        issue(i + 3, st);  // past the last stage of the last pass: a re-read nobody consumes
+        next_stage();
         wait_two_stages();  // stage i+1 has landed
         __builtin_amdgcn_s_barrier();
     }
@@ -645,23 +653,317 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     stream_epilogue<R, NT, EPI>(a, acc, e, slot_of_row, nrows, group, r0, bias_raw);
 }
 
+// ws_consumer for blocks that cover up to 2 CONS row units.
+// The wave takes row units unit0 and, with two passes, unit0 + unit_step (each if < unit_end), one per
+// pass over the bucket's activation stages (which the producers stream `passes` <= 2 times); in a pass
+// without a unit of its own it only takes part in the barriers.  The weight ring runs on across passes: the loads that the last
+// stages of a pass issue are the first stages of the next pass's unit, so only the first pass of a
+// block starts from an empty pipeline, and a pass's epilogue runs while those loads are in flight.
+// Kept apart from ws_consumer: the second pass's code costs registers even when it does not run, so
+// blocks that make one pass use the single-pass function.
+template <int FMT, int NT, int EPI, bool PRE = false, class SlotFn>
+MOE_DEVICE void ws_consumer_two(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows, int unit0,
+                            int unit_end, int unit_step, int passes) {
+    constexpr int R = 2;
+    constexpr bool TWO = true;
+    const int lane = threadIdx.x & 63;
+    const int g = lane >> 4;
+    const int q = lane & 15;
+    const int K = a.K;
+    const int n_stages = ceil_div(K, kStageElems);
+    if (unit0 >= unit_end) {  // no unit at all: barriers only
+        for (int i = 0; i < 1 + (PRE ? 1 : 0) + passes * n_stages; ++i) __syncthreads();
+        return;
+    }
+    const uint8_t* const lds_rd = lds + (size_t)q * 256;
+    // gs: stage counted over all passes (the producers' ring slot)
+    auto b_frag = [&](int gs, int j, int t) {
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(gs & (kWsRing - 1)) * kLdsStageBytes + t * 4096 +
+                                               ((ws_chunk<FMT>(j, g) ^ q) << 4));
+    };
+    f32x4 acc[R][NT];
+    uint2 bias_raw[R];
+
+    if constexpr (FMT == FMT_BF16) {
+        // The contraction range is walked in pairs of MFMA steps (64 elements = one 128-byte
+        // line of a weight row): in a pair, lane group g takes elements 16g .. 16g+7 in the first
+        // step and 16g+8 .. 16g+15 in the second, so a lane's two 16-byte loads are adjacent and
+        // the four lane groups cover the whole line.  Ring of four pairs, loads issued three
+        // pairs (one and a half stages) ahead of their use; nothing touches a loaded value
+        // before the pair that consumes it.  Pair numbers at or past n_pad (the pair count rounded up
+        // to whole ring revolutions) mean the next pass's unit; those in between are never used and
+        // re-read pair 0.
+        constexpr int DP = 4;
+        const int n_pairs = K / 64;
+        const int n_pad = ((n_stages + 1) & ~1) * 2;
+        const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
+        auto row_ptr = [&](int unit, int r) {
+            const int row = (unit >> 1) * 64 + tile_row_in_group((unit & 1) * R + r, q);
+            return reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 16 * g);
+        };
+        const uint8_t* a_ptr[R];
+        const uint8_t* a_nxt[R];
+        u32x4 ar[DP][2][R];
+        auto load_a = [&](int slot, int pair) {
+            if constexpr (TWO) {
+                const bool nxt = pair >= n_pad;  // wave-uniform
+                const int pl = nxt ? pair - n_pad : pair;
+                const size_t off = (size_t)(pl < n_pairs ? pl : 0) * 128;
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        ar[slot][h][r] = *reinterpret_cast<const u32x4*>((nxt ? a_nxt[r] : a_ptr[r]) + off + 16 * h);
+            } else {
+                const size_t off = (size_t)(pair < n_pairs ? pair : 0) * 128;  // a padding pair re-reads pair 0 (unused)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int r = 0; r < R; ++r) ar[slot][h][r] = *reinterpret_cast<const u32x4*>(a_ptr[r] + off + 16 * h);
+            }
+        };
+        // one pass; written out once per pass instead of looped (a loop around the stage code costs the
+        // compiler's register allocation dearly), so a block has at most two passes
+        auto do_pass = [&](auto first_tag, int unit, bool more, int gs0) {
+            constexpr bool first = decltype(first_tag)::value;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                a_ptr[r] = row_ptr(unit, r);
+                if constexpr (TWO) a_nxt[r] = more ? row_ptr(unit + unit_step, r) : a_ptr[r];
+            }
+            load_bias<R>(a, e, unit >> 1, (unit & 1) * R, bias_raw);  // fetched now, used by the epilogue
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (first) {
+#pragma unroll
+                for (int i = 0; i < DP - 1; ++i) load_a(i, i);
+                if constexpr (PRE) __syncthreads();
+                __syncthreads();
+            }
+            // one stage = two pairs; `ss` (stage parity) fixes the ring slots at compile time
+            auto stage = [&](auto ss_tag, int st) {
+                constexpr int ss = decltype(ss_tag)::value;
+#pragma unroll
+                for (int pp = 0; pp < 2; ++pp) {
+                    constexpr int kSlots = DP;
+                    const int u = 2 * ss + pp;  // ring slot of this pair
+                    const int pair = 2 * st + pp;
+                    load_a((u + kSlots - 1) % kSlots, pair + kSlots - 1);
+                    __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three pairs ahead of their use
+                    const bool live = pair < n_pairs;   // wave-uniform; false only in the second half of a ragged stage
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        u32x4 b[NT];
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) b[t] = b_frag(gs0 + st, 2 * pp + h, t);
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const u32x4 av = live ? ar[u][h][r] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                            for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
+                        }
+                    }
+                }
+                __syncthreads();
+            };
+            const int n_even = n_stages & ~1;
+            for (int s0 = 0; s0 < n_even; s0 += 2) {
+                stage(std::integral_constant<int, 0>{}, s0);
+                stage(std::integral_constant<int, 1>{}, s0 + 1);
+            }
+            if (n_stages & 1) {
+                stage(std::integral_constant<int, 0>{}, n_even);
+                if constexpr (TWO) {  // the loads the missing second stage of this ring revolution would have issued
+                    load_a(1, 2 * (n_even + 1) + 3);
+                    load_a(2, 2 * (n_even + 1) + 4);
+                }
+            }
+            stream_epilogue<R, NT, EPI>(a, acc, e, slot_of_row, nrows, unit >> 1, (unit & 1) * R, bias_raw);
+        };
+        if constexpr (TWO) {
+            const int unit1 = unit0 + unit_step;
+            do_pass(std::true_type{}, unit0, passes > 1 && unit1 < unit_end, 0);
+            if (passes > 1) {
+                if (unit1 < unit_end) do_pass(std::false_type{}, unit1, false, n_stages);
+                else for (int i = 0; i < n_stages; ++i) __syncthreads();  // wave-uniform: no unit left for this wave
+            }
+        } else {
+            do_pass(std::true_type{}, unit0, false, 0);
+        }
+    } else {
+        // Weights: a ring of four stages (one 128-bit load per row tile and stage, issued three
+        // stages ahead of its use); scales: one word per row tile covers four stages and is
+        // fetched one group of four ahead.  Addresses are a wave-uniform base (scalar registers)
+        // plus a per-lane 32-bit offset that never changes, so a stage costs scalar arithmetic
+        // only.  Nothing touches a loaded value before the stage that consumes it: an instruction
+        // on it at load time would pin the wait for the load to the stage that issued it.
+        // Stage numbers at or past n_pad (the stage count rounded up to whole groups of four) mean the
+        // next pass's unit; those in between are never used and re-read stage 0 with scale 0.
+        constexpr int D = 4;
+        const int G = K / 32;
+        const int rem_groups = G & 3;  // MX blocks in a ragged last stage (0 = none)
+        const size_t tile_bytes = (size_t)G * 256;
+        const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
+        const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
+        const uint8_t* sbase = a.w_scales + (size_t)e * a.s_expert_stride;
+        const uint8_t* wtile[R];  // wave-uniform
+        const uint8_t* stile[R];
+        const uint8_t* wnext[R];
+        const uint8_t* snext[R];
+        const uint32_t voff_w = (uint32_t)lane * 16;
+        // ragged last stage: a lane group past the last MX block re-reads block 0 and gets scale 0
+        const uint32_t voff_w_ragged = (uint32_t)((g < rem_groups ? lane : q) * 16);
+        const uint32_t voff_s = (uint32_t)lane * 4;
+        const int n_quads = ceil_div(n_stages, 4);
+        const int n_pad = 4 * n_quads;
+        u32x4 araw[D][R];
+        uint32_t sw_cur[R], sw_nxt[R];
+        auto load_a = [&](int slot, int s) {
+            const bool nxt = TWO && s >= n_pad;  // wave-uniform
+            const int sl = nxt ? s - n_pad : s;
+            const int su = sl < n_stages ? sl : 0;
+            const bool ragged = rem_groups != 0 && su == n_stages - 1;
+            const uint32_t vo = ragged ? voff_w_ragged : voff_w;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                // non-temporal: a 1 KiB chunk is read once, by this instruction alone, so keeping its
+                // lines in L1/L2 only evicts the activation rows (measured: -5 % kernel time; the bf16
+                // path, where two instructions share each line, and the prefill kernel, where
+                // neighbouring token blocks re-read the weights, are slower with it)
+                araw[slot][r] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4*>((nxt ? wnext[r] : wtile[r]) + (size_t)su * 1024 + vo));
+        };
+        auto load_scales = [&](uint32_t (&dst)[R], int quad) {  // quad n_quads = the next pass's first
+            const bool nxt = TWO && quad >= n_quads;
+            const size_t off = (size_t)(nxt ? 0 : min(quad, n_quads - 1)) * 256;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                dst[r] = *reinterpret_cast<const uint32_t*>((nxt ? snext[r] : stile[r]) + off + voff_s);
+        };
+        // one pass; written out once per pass instead of looped (see the bf16 branch)
+        auto do_pass = [&](auto first_tag, int unit, bool more, int gs0) {
+            constexpr bool first = decltype(first_tag)::value;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const size_t tile = (size_t)(unit >> 1) * 4 + ((unit & 1) * R + r);
+                const size_t tile_n = more ? (size_t)((unit + unit_step) >> 1) * 4 + (((unit + unit_step) & 1) * R + r) : tile;
+                wtile[r] = wbase + tile * tile_bytes;
+                stile[r] = sbase + tile * stile_bytes;
+                if constexpr (TWO) {
+                    wnext[r] = wbase + tile_n * tile_bytes;
+                    snext[r] = sbase + tile_n * stile_bytes;
+                }
+            }
+            load_bias<R>(a, e, unit >> 1, (unit & 1) * R, bias_raw);  // fetched now, used by the epilogue
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (first) {
+                load_scales(sw_cur, 0);
+#pragma unroll
+                for (int i = 0; i < D - 1; ++i) load_a(i, i);
+                if constexpr (PRE) __syncthreads();
+                __syncthreads();
+            }
+            // stage st, the i-th of its group of four (i fixes ring slot and scale byte at compile time)
+            auto stage = [&](auto i_tag, int st) {
+                constexpr int i = decltype(i_tag)::value;
+                load_a((i + D - 1) % D, st + D - 1);
+                __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three stages ahead of their use
+                const bool live = !(rem_groups != 0 && st == n_stages - 1 && g >= rem_groups);
+                float sc[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu) : 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    u32x4 b[NT];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) b[t] = b_frag(gs0 + st, j, t);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        uint32_t d[4];
+                        mxfp4_dword_to_bf16x8(araw[i][r][j], sc[r], d);
+                        const u32x4 av = {d[0], d[1], d[2], d[3]};
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
+                    }
+                }
+                __syncthreads();
+            };
+            const int full_quads = n_stages / 4;
+            for (int qd = 0; qd < full_quads; ++qd) {
+                load_scales(sw_nxt, qd + 1);
+                stage(std::integral_constant<int, 0>{}, 4 * qd + 0);
+                stage(std::integral_constant<int, 1>{}, 4 * qd + 1);
+                stage(std::integral_constant<int, 2>{}, 4 * qd + 2);
+                stage(std::integral_constant<int, 3>{}, 4 * qd + 3);
+#pragma unroll
+                for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
+            }
+            // the last, partial group of four (wave-uniform conditions; its weights are already in the
+            // ring); the stages it lacks still issue their loads, which belong to the next pass
+            const int tail = n_stages - 4 * full_quads;
+            if constexpr (TWO) {
+                if (tail > 0) {
+                    load_scales(sw_nxt, n_quads);
+                    stage(std::integral_constant<int, 0>{}, 4 * full_quads + 0);
+                    if (tail > 1) stage(std::integral_constant<int, 1>{}, 4 * full_quads + 1);
+                    else load_a(0, 4 * full_quads + 4);
+                    if (tail > 2) stage(std::integral_constant<int, 2>{}, 4 * full_quads + 2);
+                    else load_a(1, 4 * full_quads + 5);
+                    load_a(2, 4 * full_quads + 6);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
+                }
+            } else {
+                if (tail > 0) stage(std::integral_constant<int, 0>{}, 4 * full_quads + 0);
+                if (tail > 1) stage(std::integral_constant<int, 1>{}, 4 * full_quads + 1);
+                if (tail > 2) stage(std::integral_constant<int, 2>{}, 4 * full_quads + 2);
+            }
+            stream_epilogue<R, NT, EPI>(a, acc, e, slot_of_row, nrows, unit >> 1, (unit & 1) * R, bias_raw);
+        };
+        if constexpr (TWO) {
+            const int unit1 = unit0 + unit_step;
+            do_pass(std::true_type{}, unit0, passes > 1 && unit1 < unit_end, 0);
+            if (passes > 1) {
+                if (unit1 < unit_end) do_pass(std::false_type{}, unit1, false, n_stages);
+                else for (int i = 0; i < n_stages; ++i) __syncthreads();  // wave-uniform: no unit left for this wave
+            }
+        } else {
+            do_pass(std::true_type{}, unit0, false, 0);
+        }
+    }
+}
+
+template <int FMT, int NT, int EPI, bool PRE, bool TWO, class SlotFn>
+MOE_DEVICE void ws_consume_units(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows,
+                                 int unit0, int unit_end, int unit_step, int passes) {
+    if constexpr (TWO) ws_consumer_two<FMT, NT, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit0, unit_end, unit_step, passes);
+    else ws_consumer<FMT, NT, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit0, unit0 < unit_end);
+}
+
 // One token block: the producer or consumer role of this wave, for the block's token-tile count.
-template <int FMT, int EPI, int CONS, int PROD, bool PRE = false, class RowFn, class SlotFn>
-MOE_DEVICE void ws_token_block(const ExpertGemmArgs& a, uint8_t* lds, int wave, int unit, bool active, int e,
-                               RowFn act_row, SlotFn slot_of_row, int nrows) {
+// u0, u1: the block's row units [u0, u1), walked in passes of CONS units.
+template <int FMT, int EPI, int CONS, int PROD, bool PRE = false, bool TWO = false, class RowFn, class SlotFn>
+MOE_DEVICE void ws_token_block(const ExpertGemmArgs& a, uint8_t* lds, int wave, int u0, int u1, int e, RowFn act_row,
+                               SlotFn slot_of_row, int nrows) {
     const int nt = (nrows + 15) >> 4;  // block-uniform
+    const int passes = TWO ? min(2, max(1, ceil_div(u1 - u0, CONS))) : 1;
     if (wave >= CONS) {
         const int p = wave - CONS;
         if constexpr (PRE) __syncthreads();  // no direct-to-LDS load is in flight yet
-        if (nt == 4) ws_producer<FMT, 4, PROD>(a, lds, act_row, nrows, p);
-        else if (nt == 3) ws_producer<FMT, 3, PROD>(a, lds, act_row, nrows, p);
-        else if (nt == 2) ws_producer<FMT, 2, PROD>(a, lds, act_row, nrows, p);
-        else ws_producer<FMT, 1, PROD>(a, lds, act_row, nrows, p);
+        if (nt == 4) ws_producer<FMT, 4, PROD>(a, lds, act_row, nrows, p, passes);
+        else if (nt == 3) ws_producer<FMT, 3, PROD>(a, lds, act_row, nrows, p, passes);
+        else if (nt == 2) ws_producer<FMT, 2, PROD>(a, lds, act_row, nrows, p, passes);
+        else ws_producer<FMT, 1, PROD>(a, lds, act_row, nrows, p, passes);
     } else {
-        if (nt == 4) ws_consumer<FMT, 4, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
-        else if (nt == 3) ws_consumer<FMT, 3, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
-        else if (nt == 2) ws_consumer<FMT, 2, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
-        else ws_consumer<FMT, 1, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit, active);
+        if (nt == 4) ws_consume_units<FMT, 4, EPI, PRE, TWO>(a, lds, e, slot_of_row, nrows, u0 + wave, u1, CONS, passes);
+        else if (nt == 3) ws_consume_units<FMT, 3, EPI, PRE, TWO>(a, lds, e, slot_of_row, nrows, u0 + wave, u1, CONS, passes);
+        else if (nt == 2) ws_consume_units<FMT, 2, EPI, PRE, TWO>(a, lds, e, slot_of_row, nrows, u0 + wave, u1, CONS, passes);
+        else ws_consume_units<FMT, 1, EPI, PRE, TWO>(a, lds, e, slot_of_row, nrows, u0 + wave, u1, CONS, passes);
     }
 }
 
@@ -674,13 +976,11 @@ MOE_DEVICE void ws_block_coords(const ExpertGemmArgs& a, int& item, int& rb) {
     rb = a.xcd_tiles ? (blockIdx.x >> 3) % n_rb : blockIdx.x % n_rb;
 }
 
-// the row units of the weight matrix are spread evenly over the row blocks
-MOE_DEVICE void ws_row_unit(const ExpertGemmArgs& a, int rb, int wave, int& unit, bool& active) {
+// the row units of the weight matrix are spread evenly over the row blocks: block rb takes [u0, u1)
+MOE_DEVICE void ws_row_units(const ExpertGemmArgs& a, int rb, int& u0, int& u1) {
     const int units = a.rows / 32;
-    const int u0 = (int)((long long)rb * units / a.row_blocks);
-    const int u1 = (int)((long long)(rb + 1) * units / a.row_blocks);
-    unit = u0 + wave;
-    active = unit < u1;
+    u0 = (int)((long long)rb * units / a.row_blocks);
+    u1 = (int)((long long)(rb + 1) * units / a.row_blocks);
 }
 
 // Token blocks from the tile map written by the bucketing kernel.
@@ -696,11 +996,10 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
     const int e = a.tile_expert[tile];
     const int row0 = a.tile_row0[tile];
     const int nrows = a.tile_rows[tile];
-    int unit;
-    bool active;
-    ws_row_unit(a, rb, wave, unit, active);
+    int u0, u1;
+    ws_row_units(a, rb, u0, u1);
     ws_token_block<FMT, EPI, CONS, PROD>(
-        a, lds, wave, unit, active, e, [&](int i) { return a.gather ? a.tokens_flat[row0 + i] : row0 + i; },
+        a, lds, wave, u0, u1, e, [&](int i) { return a.gather ? a.tokens_flat[row0 + i] : row0 + i; },
         [&](int i) { return row0 + i; }, nrows);
 }
 
@@ -719,7 +1018,8 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
 constexpr int kDirectMaxAssign = 4096;  // 64 chunks of 64: one lane per chunk in the prefix sum
 constexpr int kDirectMaxRows = 2048;    // longest bucket the LDS list holds
 
-template <int FMT, int EPI, int CONS, int PROD>
+// TWO: blocks cover up to 2 CONS row units, in two passes over the bucket's activations.
+template <int FMT, int EPI, int CONS, int PROD, bool TWO>
 __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) void expert_stream_direct_kernel(ExpertGemmArgs a) {
     constexpr int WAVES = CONS + PROD;
     constexpr int P = (64 + WAVES - 1) / WAVES;  // chunks per wave
@@ -732,9 +1032,8 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_chunks = (a.n_assign + 63) >> 6;
-    int unit;
-    bool active;
-    ws_row_unit(a, rb, wave, unit, active);
+    int u0, u1;
+    ws_row_units(a, rb, u0, u1);
     int n_bucket;
     {
         // this wave's chunks of the assignment list
@@ -777,14 +1076,15 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
     // code; what is left are whole blocks of 64 rows, run by a loop that holds the four-tile variant
     // only (a loop around all tile-count variants costs every variant 30 registers per lane).
     const int first = n_bucket - ((n_bucket - 1) & ~63);
-    ws_token_block<FMT, EPI, CONS, PROD, true>(
-        a, lds, wave, unit, active, e, [&](int i) { return a.gather ? token_of(bucket[i]) : bucket[i]; },
+    ws_token_block<FMT, EPI, CONS, PROD, true, TWO>(
+        a, lds, wave, u0, u1, e, [&](int i) { return a.gather ? token_of(bucket[i]) : bucket[i]; },
         [&](int i) { return bucket[i]; }, first);
+    const int passes = TWO ? min(2, max(1, ceil_div(u1 - u0, CONS))) : 1;
     for (int row0 = first; row0 < n_bucket; row0 += 64) {
         auto act_row = [&](int i) { return a.gather ? token_of(bucket[row0 + i]) : bucket[row0 + i]; };
         auto slot_of_row = [&](int i) { return bucket[row0 + i]; };
-        if (wave >= CONS) ws_producer<FMT, 4, PROD>(a, lds, act_row, 64, wave - CONS);
-        else ws_consumer<FMT, 4, EPI>(a, lds, e, slot_of_row, 64, unit, active);
+        if (wave >= CONS) ws_producer<FMT, 4, PROD>(a, lds, act_row, 64, wave - CONS, passes);
+        else ws_consume_units<FMT, 4, EPI, false, TWO>(a, lds, e, slot_of_row, 64, u0 + wave, u1, CONS, passes);
     }
 }
 
@@ -1033,12 +1333,26 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             if (a.n_assign > kDirectMaxAssign || a.assign_div <= 0 || a.assign_div > 8 || a.n_experts <= 0) return MOE_ERR_LIMIT;
             ExpertGemmArgs b = a;
             const int cons = a.waves_per_block == 1 ? 12 : 10;
-            b.row_blocks = max(a.row_blocks, ceil_div(a.rows / 32, cons));
+            // a block covers at most `cons` row units per pass; MXFP4 blocks may make two passes (the
+            // second pass's code would cost the bf16 stage loops registers they do not have)
+            const int units = a.rows / 32;
+            b.row_blocks = max(a.row_blocks, ceil_div(units, (FMT == FMT_MXFP4 ? 2 : 1) * cons));
+            const bool two = ceil_div(units, b.row_blocks) > cons;
             dim3 grid(ceil_div(a.n_experts, 8) * 8 * b.row_blocks);
+            if constexpr (FMT == FMT_MXFP4) {
+                if (two && cons == 12) {
+                    hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 12, 2, true>), grid, dim3(896), 0, stream, b);
+                    return launch_status();
+                }
+                if (two) {
+                    hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 10, 2, true>), grid, dim3(768), 0, stream, b);
+                    return launch_status();
+                }
+            }
             if (cons == 12) {
-                hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 12, 2>), grid, dim3(896), 0, stream, b);
+                hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 12, 2, false>), grid, dim3(896), 0, stream, b);
             } else {
-                hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 10, 2>), grid, dim3(768), 0, stream, b);
+                hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 10, 2, false>), grid, dim3(768), 0, stream, b);
             }
         } else if (a.waves_per_block == 16) {
             ExpertGemmArgs b = a;
