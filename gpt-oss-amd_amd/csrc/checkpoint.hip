@@ -10,6 +10,7 @@
 
 #include <algorithm>
 #include <new>
+#include <initializer_list>
 #include <string>
 #include <vector>
 
@@ -82,33 +83,40 @@ int index_bin(moe_ckpt* ck, int payload_dtype) {
     if (V > (1ll << 24) || H > (1ll << 20) || E > 4096 || I > (1ll << 20) || L > 4096 || hd > 4096 || nq > 4096 ||
         nkv > 4096)
         return MOE_ERR_PARSE;
-    const long long qkv = hd * nq + 2 * hd * nkv;
+    const long long qkv = hd * nq + 2 * hd * nkv;  // at most 3 * 2^24 under the limits above
+    // The header's fields come from the file: every product and the running sum are checked, so a
+    // header whose sizes do not fit 63 bits is a parse error instead of a wrapped offset.
+    bool overflow = false;
     long long pos = 0;
-    pos += V * H;                // token_embedding_table
-    pos += V * H;                // out (unembedding)
-    pos += L * H;                // rms_attn_w
-    const long long rms_ffn = pos;
-    pos += L * H;                // rms_ffn_w
-    pos += H;                    // rms_out_w
-    pos += L * H * qkv;          // w_qkv
-    pos += L * qkv;              // b_qkv
-    pos += L * (hd * nq) * H;    // w_o
-    pos += L * H;                // b_o
-    pos += L * nq;               // attn_sinks
-    const long long w_router = pos;
-    pos += L * H * E;
-    const long long b_router = pos;
-    pos += L * E;
-    const long long w_mlp1 = pos;
-    pos += L * E * 2 * I * H;
-    const long long b_mlp1 = pos;
-    pos += L * E * 2 * I;
-    const long long w_mlp2 = pos;
-    pos += L * E * H * I;
-    const long long b_mlp2 = pos;
-    pos += L * E * H;
+    auto take = [&](std::initializer_list<long long> factors) {  // returns the offset of the tensor it appends
+        const long long at = pos;
+        long long n = 1;
+        for (const long long f : factors) overflow |= __builtin_mul_overflow(n, f, &n);
+        overflow |= __builtin_add_overflow(pos, n, &pos);
+        return at;
+    };
+    take({V, H});                                     // token_embedding_table
+    take({V, H});                                     // out (unembedding)
+    take({L, H});                                     // rms_attn_w
+    const long long rms_ffn = take({L, H});           // rms_ffn_w
+    take({H});                                        // rms_out_w
+    take({L, H, qkv});                                // w_qkv
+    take({L, qkv});                                   // b_qkv
+    take({L, hd * nq, H});                            // w_o
+    take({L, H});                                     // b_o
+    take({L, nq});                                    // attn_sinks
+    const long long w_router = take({L, H, E});
+    const long long b_router = take({L, E});
+    const long long w_mlp1 = take({L, E, 2 * I, H});
+    const long long b_mlp1 = take({L, E, 2 * I});
+    const long long w_mlp2 = take({L, E, H, I});
+    const long long b_mlp2 = take({L, E, H});
     const size_t eb = dtype_bytes(payload_dtype);
-    if (ck->map_bytes != sizeof(moe_ckpt_config) + (size_t)pos * eb) return MOE_ERR_SHAPE;
+    long long payload_bytes = 0, file_bytes = 0;
+    overflow |= __builtin_mul_overflow(pos, (long long)eb, &payload_bytes);
+    overflow |= __builtin_add_overflow(payload_bytes, (long long)sizeof(moe_ckpt_config), &file_bytes);
+    if (overflow) return MOE_ERR_PARSE;
+    if (ck->map_bytes != (size_t)file_bytes) return MOE_ERR_SHAPE;
 
     struct Slot {
         int which;
@@ -131,6 +139,7 @@ int index_bin(moe_ckpt* ck, int payload_dtype) {
             for (int i = 0; i < s.rank; ++i) t.shape[i] = s.shape[i];
             t.offset = sizeof(moe_ckpt_config) + (size_t)(s.base + l * s.per_layer) * eb;
             t.bytes = (size_t)s.per_layer * eb;
+            if (t.offset > ck->map_bytes || t.bytes > ck->map_bytes - t.offset) return MOE_ERR_SHAPE;
             ck->layer_index[(size_t)l * MOE_T_COUNT + s.which] = (int)ck->tensors.size();
             ck->tensors.push_back(t);
         }

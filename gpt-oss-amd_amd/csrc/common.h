@@ -153,7 +153,11 @@ MOE_DEVICE float swiglu(float gate, float up, float alpha, float limit) {
     up = up < -limit ? -limit : up;
     // exp through the hardware exp2 (relative error ~1e-6, far inside the 1e-2 output tolerance;
     // the reference's own GPU kernel uses __expf as well, src/hip/moe.hip:189)
+#ifdef MOE_EXP_RCP
+    const float sig = __builtin_amdgcn_rcpf(1.0f + __expf(-alpha * gate));
+#else
     const float sig = 1.0f / (1.0f + __expf(-alpha * gate));
+#endif
     return (gate * sig) * (up + 1.0f);
 }
 

@@ -1358,7 +1358,11 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             ExpertGemmArgs b = a;
             b.row_blocks = ceil_div(a.rows / 64, 4);
             dim3 grid(ceil_div(a.max_tiles, 8) * 8 * b.row_blocks);  // every XCD gets whole token blocks
+#ifdef MOE_EXP_1BLK
+            hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 40 * 1024, stream, b);
+#else
             hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 0, stream, b);
+#endif
         } else if (a.waves_per_block == 0) {
             ExpertGemmArgs b = a;
             b.row_blocks = max(a.row_blocks, ceil_div(a.rows / 32, 10));

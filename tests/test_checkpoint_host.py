@@ -85,6 +85,14 @@ def test_bin_rejects_wrong_files(ck, tmp_path):
     assert code_of(raw[:40]) == -8               # header cut short
     assert code_of(struct.pack("<i", -5) + raw[4:]) == -8   # nonsense config
     assert code_of(raw, dtype=7) == -5
+    # every field inside its own limit, but the tensor sizes multiply out past 63 bits: a parse error,
+    # not an offset that wrapped around to something that happens to match the file size
+    huge = dict(cfg, vocab_size=1 << 24, hidden_size=1 << 20, num_experts=4096, experts_per_token=4,
+                intermediate_size=1 << 20, num_hidden_layers=4096, head_dim=4096, num_attention_heads=4096,
+                num_key_value_heads=4096)
+    header = b"".join(struct.pack("<i" if isinstance(huge[k], int) else "<f", huge[k]) for k in ckptgen.CONFIG_KEYS)
+    assert code_of(header + raw[len(header):]) == -8
+    assert code_of(header) == -8
     with pytest.raises(Exception) as e:
         ck.Checkpoint.open_bin(tmp_path / "does_not_exist.bin")
     assert e.value.code == -7
