@@ -56,7 +56,7 @@ struct BlockWorkspace {
     int* tokens_flat;      // [A]
     float* weights_flat;   // [A]
     int* slot_of;          // [A]
-    int* tile_expert;      // [max_tiles]
+    int* tile_expert;      // [2][max_tiles]: the token-block map in two orders (bucket.hip)
     int* tile_row0;
     int* tile_rows;
     int* n_tiles;          // [1]
@@ -82,9 +82,9 @@ struct BlockWorkspace {
         weights_flat = static_cast<float*>(take(A * 4));
         slot_of = static_cast<int*>(take(A * 4));
         max_tiles = tile_map_capacity((int)A, E, kStreamTileTokens);
-        tile_expert = static_cast<int*>(take((size_t)max_tiles * 4));
-        tile_row0 = static_cast<int*>(take((size_t)max_tiles * 4));
-        tile_rows = static_cast<int*>(take((size_t)max_tiles * 4));
+        tile_expert = static_cast<int*>(take((size_t)2 * max_tiles * 4));
+        tile_row0 = static_cast<int*>(take((size_t)2 * max_tiles * 4));
+        tile_rows = static_cast<int*>(take((size_t)2 * max_tiles * 4));
         n_tiles = static_cast<int*>(take(4));
         h_by_slot = static_cast<uint16_t*>(take(A * I * 2));
         y_by_slot = static_cast<float*>(take(A * H * 4));
@@ -185,8 +185,8 @@ int moe_bucket_by_expert(const int* topk_i, const float* topk_v, int B, int K, i
                          int* tokens_flat, float* weights_flat, int* slot_of, moe_stream_t stream) {
     if (!topk_i || !topk_v || !expert_offsets || !tokens_flat || !weights_flat) return MOE_ERR_NULL;
     if (B <= 0 || K <= 0 || E <= 0) return MOE_ERR_SHAPE;
-    if (E > 1024 || (long long)B * K > 0x7FFFFFFFll / 4) return MOE_ERR_LIMIT;
-    TileMap none{nullptr, nullptr, nullptr, nullptr, 0, 0};
+    if (E > 1024 || K > 8 || (long long)B * K > 0x7FFFFFFFll / 4) return MOE_ERR_LIMIT;
+    TileMap none{nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
     return launch_bucket(topk_i, topk_v, B, K, E, expert_offsets, tokens_flat, weights_flat, slot_of, none,
                          as_stream(stream));
 }
@@ -400,6 +400,7 @@ struct ExpertPlan {
     ExpertGemmArgs g{};
     bool prefill, direct;
     int est_tiles, n_cus;
+    int second_map;  // index of the token-block map in bucket order inside the map arrays
 
     ExpertPlan(const moe_block_params* p_, const BlockWorkspace& ws, bool prefill_, bool direct_, int tile_tokens,
                int max_tiles)
@@ -422,6 +423,7 @@ struct ExpertPlan {
         }
         est_tiles = direct ? E : std::max(ceil_div(T * K, tile_tokens), std::min(E, T * K));
         n_cus = device_cu_count();
+        second_map = ws.max_tiles;
     }
     // Decode-sized buckets (producer/consumer kernel, one block per CU): 10 or 12 consumer waves of
     // 32 rows each.  Blocks run in rounds of one per CU, so the cheaper choice is the one with the
@@ -499,6 +501,15 @@ struct ExpertPlan {
         a.act = act;
         a.gather = 0;
         a.out = out;
+        // Measured at 4096 tokens: the gate/up GEMM is up to 9 % faster with the partial token blocks last
+        // (largest first: the launch's tail is made of short blocks); the down GEMM is 2 % faster in bucket
+        // order, where a partial block runs next to full blocks of its expert and finds the expert's weights
+        // on their way through the caches.
+        if (!direct) {
+            a.tile_expert += second_map;
+            a.tile_row0 += second_map;
+            a.tile_rows += second_map;
+        }
         // measured: the down GEMM gains 4-10 % from keeping a token block on one XCD (its input rows were
         // written by the gate/up launch just before), the gate/up GEMM loses up to 2 %
         a.xcd_tiles = 1;
@@ -574,7 +585,7 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     const int tile_tokens = prefill ? kPrefillTileTokens : kStreamTileTokens;
     const int max_tiles = tile_map_capacity(T * K, E, tile_tokens);  // <= ws.max_tiles (sized for 64)
     if (!direct) {
-        TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles};
+        TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles, ws.max_tiles};
         rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat,
                            ws.slot_of, map, stream);
         if (rc) return rc;
@@ -681,7 +692,7 @@ int moe_block_down_gemm(const moe_block_params* caller, const moe_bf16_t* h_by_a
     const ExpertPlan plan(p, ws, prefill, direct, tile_tokens, max_tiles);
     if (direct) return launch_expert_stream(plan.down(h_by_assignment, y_by_assignment), 1, stream);
     // rows by slot: bucket, bring the caller's rows into slot order, multiply, bring the result back
-    TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles};
+    TileMap map{ws.tile_expert, ws.tile_row0, ws.tile_rows, ws.n_tiles, tile_tokens, max_tiles, ws.max_tiles};
     rc = launch_bucket(p->topk_i, p->topk_v, T, K, E, ws.expert_offsets, ws.tokens_flat, ws.weights_flat, ws.slot_of,
                        map, stream);
     if (rc) return rc;

@@ -9,98 +9,173 @@
 
 namespace moe {
 
-// grid = E blocks (one expert each), block = 1024 threads, dynamic LDS = (E + 32) ints.
+// Copies of the histogram in LDS: a wave's atomic adds go to random experts, and adds of several
+// lanes to one counter run one after the other; with one copy per lane (mod kHistCopies, the copy
+// index being the bank) two lanes meet only when they are 32 apart.
+constexpr int kHistCopies = 32;
+static int hist_copies(int E) { return E <= 256 ? kHistCopies : E <= 512 ? 16 : 8; }
+
+// grid = E blocks (one expert each), block = 1024 threads, dynamic LDS = (E * copies + E + 32) ints.
+// Tile map order: every full tile first (ascending expert), then the experts' partial last tiles from
+// the largest to the smallest (equal sizes: ascending expert).  An expert kernel that takes tiles in
+// this order runs its shortest blocks last, next to compute units that have already run out of work.
+// With map.second > 0 the same tiles are listed a second time, from index map.second of the three
+// arrays, in bucket order (an expert's tiles together, the partial one last).
 __global__ __launch_bounds__(1024) void bucket_kernel(const int* __restrict__ topk_i,
                                                       const float* __restrict__ topk_v, int T, int K, int E,
-                                                      int* __restrict__ expert_offsets,
+                                                      int copies, int* __restrict__ expert_offsets,
                                                       int* __restrict__ tokens_flat,
                                                       float* __restrict__ weights_flat,
                                                       int* __restrict__ slot_of, TileMap map) {
     extern __shared__ int lds[];
-    int* hist = lds;           // [E]
-    int* wave_cnt = lds + E;   // [16]
-    int* scal = lds + E + 16;  // [0] rows before this expert, [1] tiles before this expert
+    int* hist = lds;                  // [E]
+    int* wave_cnt = lds + E;          // [16]
+    int* scal = lds + E + 16;         // [0] rows before this expert, [1] full tiles before it, [2] full tiles in all,
+                                      // [3] partial tiles ahead of this expert's (by size), [4] partial tiles in all,
+                                      // [5] partial tiles of the experts before this one
+    int* hist_c = lds + E + 32;       // [E][copies]
     const int e = blockIdx.x;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int A = T * K;
 
-    for (int i = tid; i < E; i += blockDim.x) hist[i] = 0;
-    if (tid < 2) scal[tid] = 0;
+    for (int i = tid; i < E * copies; i += blockDim.x) hist_c[i] = 0;
+    if (tid < 8) scal[tid] = 0;
     __syncthreads();
-    for (int a = tid; a < A; a += blockDim.x) {
-        const int id = topk_i[a];
-        if ((unsigned)id < (unsigned)E) atomicAdd(&hist[id], 1);
+    const int my_copy = tid & (copies - 1);
+    // eight loads per thread in flight: the pass costs memory round trips, not adds
+    for (int a0 = tid; a0 < A; a0 += 8 * 1024) {
+        int id[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) id[u] = a0 + u * 1024 < A ? topk_i[a0 + u * 1024] : -1;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if ((unsigned)id[u] < (unsigned)E) atomicAdd(&hist_c[id[u] * copies + my_copy], 1);
+    }
+    __syncthreads();
+    for (int i = tid; i < E; i += blockDim.x) {
+        int c = 0;
+        for (int j = 0; j < copies; ++j) c += hist_c[i * copies + ((j + i) & (copies - 1))];  // rotated: no common bank
+        hist[i] = c;
     }
     __syncthreads();
     const int nb = map.tile_tokens;
+    const int my_cnt = hist[e];
     {
-        int rows_before = 0, tiles_before = 0;
-        for (int i = tid; i < e; i += blockDim.x) {
+        const int my_rem = nb > 0 ? my_cnt % nb : 0;
+        int rows_before = 0, full_before = 0, full_all = 0, part_ahead = 0, part_all = 0, part_before = 0;
+        for (int i = tid; i < E; i += blockDim.x) {
             const int c = hist[i];
-            rows_before += c;
-            if (nb > 0) tiles_before += (c + nb - 1) / nb;
+            if (i < e) rows_before += c;
+            if (nb > 0) {
+                const int full = c / nb, rem = c - full * nb;
+                full_all += full;
+                if (i < e) full_before += full;
+                if (rem > 0) {
+                    part_all += 1;
+                    if (i < e) part_before += 1;
+                    if (rem > my_rem || (rem == my_rem && i < e)) part_ahead += 1;
+                }
+            }
         }
-        if (rows_before) atomicAdd(&scal[0], rows_before);
-        if (tiles_before) atomicAdd(&scal[1], tiles_before);
+        // wave sums first, one add per wave and quantity (an atomic add of a different value per lane
+        // is carried out lane by lane)
+        int sums[6] = {rows_before, full_before, full_all, part_ahead, part_all, part_before};
+        if (wave * 64 < E) {  // wave-uniform: later waves hold zeros
+#pragma unroll
+            for (int i = 0; i < 6; ++i) {
+                const int total = wave_sum(sums[i]);
+                if (lane == 0 && total) atomicAdd(&scal[i], total);
+            }
+        }
     }
     __syncthreads();
     const int my_off = scal[0];
-    const int my_cnt = hist[e];
-    const int my_tile0 = scal[1];
     if (tid == 0) {
         expert_offsets[e] = my_off;
         if (e == E - 1) expert_offsets[E] = my_off + my_cnt;
     }
     if (nb > 0) {
-        const int my_tiles = (my_cnt + nb - 1) / nb;
-        for (int j = tid; j < my_tiles; j += blockDim.x) {
-            map.tile_expert[my_tile0 + j] = e;
-            map.tile_row0[my_tile0 + j] = my_off + j * nb;
-            map.tile_rows[my_tile0 + j] = min(nb, my_cnt - j * nb);
+        const int my_full = my_cnt / nb;
+        const int my_rem = my_cnt - my_full * nb;
+        for (int j = tid; j < my_full; j += blockDim.x) {
+            map.tile_expert[scal[1] + j] = e;
+            map.tile_row0[scal[1] + j] = my_off + j * nb;
+            map.tile_rows[scal[1] + j] = nb;
         }
-        if (e == E - 1 && tid == 0) *map.n_tiles = my_tile0 + my_tiles;
+        if (my_rem > 0 && tid == 0) {
+            const int at = scal[2] + scal[3];
+            map.tile_expert[at] = e;
+            map.tile_row0[at] = my_off + my_full * nb;
+            map.tile_rows[at] = my_rem;
+        }
+        if (map.second > 0) {  // the same tiles in bucket order: an expert's tiles together, its partial one last
+            const int first = map.second + scal[1] + scal[5];
+            for (int j = tid; j < my_full + (my_rem > 0); j += blockDim.x) {
+                map.tile_expert[first + j] = e;
+                map.tile_row0[first + j] = my_off + j * nb;
+                map.tile_rows[first + j] = min(nb, my_cnt - j * nb);
+            }
+        }
+        if (e == E - 1 && tid == 0) *map.n_tiles = scal[2] + scal[4];
     }
 
-    // ordered compaction: tokens visited in ascending id, blockDim tokens per step
+    // ordered compaction: tokens visited in ascending id, 1024 tokens per step; the ids of four steps
+    // are fetched together (K <= 8 per token)
     int base = my_off;
-    for (int t0 = 0; t0 < T; t0 += blockDim.x) {
-        const int t = t0 + tid;
-        int mk = -1;
-        if (t < T) {
-            for (int k = 0; k < K; ++k)
-                if (topk_i[(size_t)t * K + k] == e) {
-                    mk = k;
-                    break;
-                }
+    for (int t00 = 0; t00 < T; t00 += 4 * 1024) {
+        int mk4[4];
+        float wv4[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int t = t00 + u * 1024 + tid;
+            int ids[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) ids[k] = (t < T && k < K) ? topk_i[(size_t)t * K + k] : -1;
+            int mk = -1;
+#pragma unroll
+            for (int k = 7; k >= 0; --k) mk = ids[k] == e ? k : mk;  // the first k that names this expert
+            mk4[u] = mk;
         }
-        const unsigned long long ballot = __ballot(mk >= 0);
-        const int prefix = __popcll(ballot & ((1ull << lane) - 1ull));
-        if (lane == 0) wave_cnt[wave] = __popcll(ballot);
-        __syncthreads();
-        int wave_base = 0, total = 0;
-        const int n_waves = blockDim.x >> 6;
-        for (int w = 0; w < n_waves; ++w) {
-            const int c = wave_cnt[w];
-            if (w < wave) wave_base += c;
-            total += c;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {  // the matching routing weights, again before anything waits
+            const int t = t00 + u * 1024 + tid;
+            wv4[u] = mk4[u] >= 0 ? topk_v[(size_t)t * K + mk4[u]] : 0.f;
         }
-        if (mk >= 0) {
-            const int dst = base + wave_base + prefix;
-            tokens_flat[dst] = t;
-            weights_flat[dst] = topk_v[(size_t)t * K + mk];
-            if (slot_of) slot_of[(size_t)t * K + mk] = dst;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (t00 + u * 1024 >= T) break;  // block-uniform
+            const int t = t00 + u * 1024 + tid;
+            const int mk = mk4[u];
+            const unsigned long long ballot = __ballot(mk >= 0);
+            const int prefix = __popcll(ballot & ((1ull << lane) - 1ull));
+            if (lane == 0) wave_cnt[wave] = __popcll(ballot);
+            __syncthreads();
+            int wave_base = 0, total = 0;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) {
+                const int c = wave_cnt[w];
+                if (w < wave) wave_base += c;
+                total += c;
+            }
+            if (mk >= 0) {
+                const int dst = base + wave_base + prefix;
+                tokens_flat[dst] = t;
+                weights_flat[dst] = wv4[u];
+                if (slot_of) slot_of[(size_t)t * K + mk] = dst;
+            }
+            base += total;
+            __syncthreads();
         }
-        base += total;
-        __syncthreads();
     }
 }
 
 int launch_bucket(const int* topk_i, const float* topk_v, int T, int K, int E, int* expert_offsets,
                   int* tokens_flat, float* weights_flat, int* slot_of, TileMap map, hipStream_t stream) {
-    hipLaunchKernelGGL(bucket_kernel, dim3(E), dim3(1024), (size_t)(E + 32) * sizeof(int), stream, topk_i, topk_v,
-                       T, K, E, expert_offsets, tokens_flat, weights_flat, slot_of, map);
+    const int copies = hist_copies(E);
+    hipLaunchKernelGGL(bucket_kernel, dim3(E), dim3(1024), (size_t)(E * copies + E + 32) * sizeof(int), stream, topk_i,
+                       topk_v, T, K, E, copies, expert_offsets, tokens_flat, weights_flat, slot_of, map);
     return launch_status();
 }
 

@@ -121,6 +121,13 @@ MOE_DEVICE float wave_sum(float v) {
     return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
 }
 
+MOE_DEVICE int wave_sum(int v) {
+#define MOE_STEP(C, M) v += (int)dpp_move<C, M>(0u, (uint32_t)v);
+    MOE_DPP_STEPS(MOE_STEP)
+#undef MOE_STEP
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // for v >= 0
 MOE_DEVICE float wave_max_nonneg(float v) {
 #define MOE_STEP(C, M) v = fmaxf(v, __uint_as_float(dpp_move<C, M>(0u, __float_as_uint(v))));
@@ -151,13 +158,11 @@ MOE_DEVICE float swiglu(float gate, float up, float alpha, float limit) {
     gate = gate > limit ? limit : gate;
     up = up > limit ? limit : up;
     up = up < -limit ? -limit : up;
-    // exp through the hardware exp2 (relative error ~1e-6, far inside the 1e-2 output tolerance;
-    // the reference's own GPU kernel uses __expf as well, src/hip/moe.hip:189)
-#ifdef MOE_EXP_RCP
-    const float sig = __builtin_amdgcn_rcpf(1.0f + __expf(-alpha * gate));
-#else
-    const float sig = 1.0f / (1.0f + __expf(-alpha * gate));
-#endif
+    // sigmoid through the hardware's exp2 and reciprocal (each good to one unit in the last place:
+    // relative error ~1e-7, far inside the 1e-2 output tolerance; the reference's own GPU kernel uses
+    // __expf as well, src/hip/moe.hip:189).  The IEEE division the plain expression compiles to costs
+    // ten more instructions per output, and the epilogue runs with the matrix pipe idle.
+    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(gate * (alpha * -1.44269504088896f)));
     return (gate * sig) * (up + 1.0f);
 }
 

@@ -1259,6 +1259,8 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     issue_b(0);
     load_scales(sw_cur, 0);
     load_a(0, 0);
+    uint2 bias_raw[R];  // fetched with the first stage: its latency stays off the block's tail
+    load_bias<R>(a, e, unit, 0, bias_raw);
     wait_vmcnt<0>();
     __syncthreads();
     for (int qd = 0; qd < n_quads; ++qd) {
@@ -1269,8 +1271,6 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
 #pragma unroll
         for (int r = 0; r < R; ++r) sw_cur[r] = sw_nxt[r];
     }
-    uint2 bias_raw[R];
-    load_bias<R>(a, e, unit, 0, bias_raw);
     stream_epilogue<R, NT, EPI>(a, acc, e, [&](int i) { return row0 + i; }, nrows, unit, 0, bias_raw);
 }
 
@@ -1358,11 +1358,7 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             ExpertGemmArgs b = a;
             b.row_blocks = ceil_div(a.rows / 64, 4);
             dim3 grid(ceil_div(a.max_tiles, 8) * 8 * b.row_blocks);  // every XCD gets whole token blocks
-#ifdef MOE_EXP_1BLK
-            hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 40 * 1024, stream, b);
-#else
             hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 0, stream, b);
-#endif
         } else if (a.waves_per_block == 0) {
             ExpertGemmArgs b = a;
             b.row_blocks = max(a.row_blocks, ceil_div(a.rows / 32, 10));

@@ -39,6 +39,7 @@ struct TileMap {
     int* n_tiles;   // device scalar
     int tile_tokens;  // rows per tile (NB); 0 = no map requested
     int max_tiles;    // capacity = upper bound used as grid dimension
+    int second;       // the same tiles in bucket order start at this index of the three arrays (0: not wanted)
 };
 inline int tile_map_capacity(int A, int E, int tile_tokens) { return (A + tile_tokens - 1) / tile_tokens + E; }
 

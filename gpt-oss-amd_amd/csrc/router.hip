@@ -361,15 +361,14 @@ __global__ __launch_bounds__(256) void router_finalize_kernel(const double* __re
 // grid = (ceil(T/64), ceil(E/(16*NE)), S), block = 256, dynamic LDS = 16*NE*(seg_len+8)*2 bytes;
 // seg_len % 32 == 0, H % 32 == 0.
 // ---------------------------------------------------------------------------------------------
-constexpr int kScreenDepth = 4;  // k-steps whose activation loads are in flight together
-
-template <int NE>
+// D: k-steps whose activation loads are in flight together (the kernel is a chain of memory round
+// trips: one for the router rows, then one per D k-steps of its segment).
+template <int NE, int D>
 __global__ __launch_bounds__(256) void router_screen_kernel(const float* __restrict__ x,
                                                             const uint16_t* __restrict__ w,
                                                             float* __restrict__ partial, float* __restrict__ wn2,
                                                             float* __restrict__ xn2, uint16_t* __restrict__ x_bf16,
                                                             int T, int H, int E, int seg_len) {
-    constexpr int D = kScreenDepth;
     extern __shared__ __attribute__((aligned(16))) uint16_t wl[];  // [16*NE][seg_len + 8]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -877,16 +876,29 @@ int launch_router_two_pass(const float* x, const uint16_t* w, const uint16_t* bi
     const int ne = screen_tiles(E);
     dim3 grid(ceil_div(T, 64), ceil_div(E, 16 * ne), S);
     const size_t lds = (size_t)16 * ne * (seg_len + 8) * sizeof(uint16_t);
-    if (ne == 1) {
-        hipLaunchKernelGGL((router_screen_kernel<1>), grid, dim3(256), lds, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
-                           seg_len);
-    } else if (ne == 2) {
-        hipLaunchKernelGGL((router_screen_kernel<2>), grid, dim3(256), lds, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
-                           seg_len);
-    } else {
-        hipLaunchKernelGGL((router_screen_kernel<4>), grid, dim3(256), lds, stream, x, w, partial, wn2, xn2, x_bf16, T, H, E,
-                           seg_len);
+    // the whole segment in flight where it is short enough for the registers (D * 8 per lane)
+    const int steps = seg_len / 32;
+    const int depth = steps >= 12 ? 12 : steps >= 6 ? 6 : 4;
+#define MOE_SCREEN(NE_, D_)                                                                                          \
+    hipLaunchKernelGGL((router_screen_kernel<NE_, D_>), grid, dim3(256), lds, stream, x, w, partial, wn2, xn2, x_bf16, T, H, \
+                       E, seg_len)
+#define MOE_SCREEN_NE(NE_)          \
+    if (depth == 12) {              \
+        MOE_SCREEN(NE_, 12);        \
+    } else if (depth == 6) {        \
+        MOE_SCREEN(NE_, 6);         \
+    } else {                        \
+        MOE_SCREEN(NE_, 4);         \
     }
+    if (ne == 1) {
+        MOE_SCREEN_NE(1)
+    } else if (ne == 2) {
+        MOE_SCREEN_NE(2)
+    } else {
+        MOE_SCREEN_NE(4)
+    }
+#undef MOE_SCREEN_NE
+#undef MOE_SCREEN
     int rc = launch_status();
     if (rc) return rc;
     if (between) MOE_RETURN_IF_HIP(hipEventRecord(between, stream));

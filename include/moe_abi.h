@@ -129,7 +129,7 @@ MOE_API int moe_softmax(float* x, int batch_size, int size, moe_stream_t stream)
  *   tokens_flat    [B*K]  token ids grouped by expert, ascending token id inside a group
  *   weights_flat   [B*K]  the matching topk_v entry
  *   slot_of        [B*K]  optional: position of assignment (b,k) in tokens_flat
- * E <= 1024.
+ * E <= 1024, K <= 8 (the limits of moe_topk).
  * Precondition (what moe_topk and the fused router write, and what the reference's kernels assume as
  * well): the K ids of one token are pairwise distinct and every id is in [0, E).  An id outside
  * [0, E) is dropped: it is counted in no bucket, expert_offsets[E] is then smaller than B*K, and its
