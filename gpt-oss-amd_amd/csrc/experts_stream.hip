@@ -78,6 +78,44 @@ MOE_DEVICE void stream_epilogue(const ExpertGemmArgs& a, const f32x4 (&acc)[R][N
         bv[r][2] = bf16_bits_to_f32(raw.y & 0xFFFFu);
         bv[r][3] = bf16_bits_to_f32(raw.y >> 16);
     }
+    if constexpr (EPI == EPI_ROWS_F32 && R == 4) {
+        // Four row tiles per lane: lane (q, g) holds, for its token, the four 16-byte pieces g*64 + r*16 of a
+        // 256-byte stretch of the output row, so one store instruction would touch 64 pieces that are 64 bytes
+        // apart.  A 4x4 transpose between the four lane rows (g) and the four row tiles (r), two lane-row
+        // swaps per value, leaves lane (q, g) with the pieces r*64 + g*16: a store instruction then writes
+        // 64 contiguous bytes per token (four lanes), a quarter of the write requests.
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            uint32_t v[4][4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[r][j] = __float_as_uint(acc[r][t][j] + bv[r][j]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {  // lanes 32..63 of tile r <-> lanes 0..31 of tile r + 2
+                    const auto sw = __builtin_amdgcn_permlane32_swap(v[r][j], v[r + 2][j], false, false);
+                    v[r][j] = sw[0];
+                    v[r + 2][j] = sw[1];
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r += 2) {  // odd lane rows of tile r <-> even lane rows of tile r + 1
+                    const auto sw = __builtin_amdgcn_permlane16_swap(v[r][j], v[r + 1][j], false, false);
+                    v[r][j] = sw[0];
+                    v[r + 1][j] = sw[1];
+                }
+            }
+            const int idx = t * 16 + q;
+            if (idx < nrows) {
+                float* dst = reinterpret_cast<float*>(a.out) + (size_t)slot_of_row(idx) * a.rows + group * 64 + g * 4;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    *reinterpret_cast<u32x4*>(dst + 16 * r) = u32x4{v[r][0], v[r][1], v[r][2], v[r][3]};
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int idx = t * 16 + q;
