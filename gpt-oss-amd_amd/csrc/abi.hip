@@ -646,11 +646,20 @@ int moe_block_describe(const moe_block_params* p, char* text, size_t text_bytes)
     BlockWorkspace ws(nullptr, T, H, I, E, K);
     const ExpertPlan plan(p, ws, prefill, direct, tile_tokens, tile_map_capacity(T * K, E, tile_tokens));
     auto gemm_name = [&](int rows, int epi, char* out, size_t n) {
-        int kernel = plan.pick_kernel(rows), unused = 0;
-        if (direct && fmt == MOE_WEIGHTS_MXFP4_TILED) plan.pick_two_pass(rows, &kernel, &unused);
-        if (prefill) snprintf(out, n, "expert_prefill_kernel<%d, %d, 4>", fmt, epi);
-        else snprintf(out, n, "%s<%d, %d, %d, 2>", direct ? "expert_stream_direct_kernel" : "expert_stream_ws_kernel", fmt,
-                      epi, kernel == 1 ? 12 : 10);
+        int kernel = plan.pick_kernel(rows), row_blocks = plan.pick_row_blocks(rows, kernel);
+        if (direct && fmt == MOE_WEIGHTS_MXFP4_TILED) plan.pick_two_pass(rows, &kernel, &row_blocks);
+        const int cons = kernel == 1 ? 12 : 10;
+        if (prefill) {
+            snprintf(out, n, "expert_prefill_kernel<%d, %d, 4>", fmt, epi);
+        } else if (direct) {
+            // as the launcher: at least enough row blocks for one (bf16) or two (MXFP4) passes of `cons` row units
+            const int units = rows / 32;
+            const int rb = std::max(row_blocks, ceil_div(units, (fmt == MOE_WEIGHTS_MXFP4_TILED ? 2 : 1) * cons));
+            const bool two = fmt == MOE_WEIGHTS_MXFP4_TILED && ceil_div(units, rb) > cons;
+            snprintf(out, n, "expert_stream_direct_kernel<%d, %d, %d, 2, %s>", fmt, epi, cons, two ? "true" : "false");
+        } else {
+            snprintf(out, n, "expert_stream_ws_kernel<%d, %d, %d, 2>", fmt, epi, cons);
+        }
     };
     char g1[96], g2[96];
     gemm_name(2 * I, 0, g1, sizeof(g1));
