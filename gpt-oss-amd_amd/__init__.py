@@ -85,6 +85,10 @@ SIGNATURES = {
     "moe_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "moe_scatter_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "moe_build_work_queue": (_i, [_vp, _i, _vp, _vp, _vp]),
+    "moe_count_tokens_per_expert": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
+    "moe_exclusive_scan_expert_offsets": (_i, [_vp, _vp, _i, _vp]),
+    "moe_compact_by_expert": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp]),
+    "moe_classify_and_build_queues": (_i, [_vp, _i, _i, _f, _f, _vp, _vp, _vp, _vp]),
     "moe_mlp1_swiglu": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _ll, _ll, _f, _f, _i, _i, _vp]),
     "moe_mlp2_scatter": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _ll, _ll, _i, _i, _vp]),
     "moe_mlp1_swiglu_mxfp4": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _ll, _f, _f, _i, _i, _vp]),
@@ -201,6 +205,37 @@ def bucket_by_expert(topk_i, topk_v, B, K, E, expert_offsets, tokens_flat, weigh
     _check("moe_bucket_by_expert",
            _lib.moe_bucket_by_expert(_ptr(topk_i), _ptr(topk_v), B, K, E, _ptr(expert_offsets), _ptr(tokens_flat),
                                      _ptr(weights_flat), _ptr(slot_of), _stream(stream)))
+
+
+def count_tokens_per_expert(topk_i, topk_v, B, K, out_expert, out_token, out_w, counts, E, stream=None):
+    """count_tokens_per_expert of src/hip/scheduler.hip:11-31 (counts must be zero on entry)."""
+    _check("moe_count_tokens_per_expert",
+           _lib.moe_count_tokens_per_expert(_ptr(topk_i), _ptr(topk_v), B, K, _ptr(out_expert), _ptr(out_token),
+                                            _ptr(out_w), _ptr(counts), E, _stream(stream)))
+
+
+def exclusive_scan_expert_offsets(counts, offsets, E, stream=None):
+    """exclusive_scan_expert_offsets of src/hip/scheduler.hip:33-46 (zeroes counts)."""
+    _check("moe_exclusive_scan_expert_offsets",
+           _lib.moe_exclusive_scan_expert_offsets(_ptr(counts), _ptr(offsets), E, _stream(stream)))
+
+
+def compact_by_expert(expert_ids, tokens, weights, BK, offsets, write_counters, tokens_flat, weights_flat, E,
+                      stream=None):
+    """compact_by_expert_kernel of src/hip/scheduler.hip:48-61, buckets in ascending assignment index."""
+    _check("moe_compact_by_expert",
+           _lib.moe_compact_by_expert(_ptr(expert_ids), _ptr(tokens), _ptr(weights), BK, _ptr(offsets),
+                                      _ptr(write_counters), _ptr(tokens_flat), _ptr(weights_flat), E, _stream(stream)))
+
+
+def classify_and_build_queues(expert_offsets, E, very_sparse_cutoff, heavy_factor_sparse, heavy_factor_default,
+                              wq_heavy, wq_light, stats, stream=None):
+    """classify_and_build_queues of src/hip/scheduler.hip:112-184; `stats` is a device buffer of 24 bytes
+    (four int32 and one int64: heavy_count, light_count, heavy_maxNe, active_experts, sumNe)."""
+    _check("moe_classify_and_build_queues",
+           _lib.moe_classify_and_build_queues(_ptr(expert_offsets), E, very_sparse_cutoff, heavy_factor_sparse,
+                                              heavy_factor_default, _ptr(wq_heavy), _ptr(wq_light), _ptr(stats),
+                                              _stream(stream)))
 
 
 def gather_rows(X, idx, Y, rows, H, stream=None):

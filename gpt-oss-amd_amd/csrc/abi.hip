@@ -217,6 +217,42 @@ int moe_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, 
     return MOE_OK;
 }
 
+int moe_count_tokens_per_expert(const int* topk_i, const float* topk_v, int B, int K, int* out_expert, int* out_token,
+                                float* out_w, int* counts, int E, moe_stream_t stream) {
+    if (!topk_i || !topk_v || !out_expert || !out_token || !out_w || !counts) return MOE_ERR_NULL;
+    if (B <= 0 || K <= 0 || E <= 0) return MOE_ERR_SHAPE;
+    if (E > 1024 || (long long)B * K >= (1LL << 29)) return MOE_ERR_LIMIT;
+    return launch_count_tokens_per_expert(topk_i, topk_v, B, K, out_expert, out_token, out_w, counts, E,
+                                          as_stream(stream));
+}
+
+int moe_exclusive_scan_expert_offsets(int* counts, int* offsets, int E, moe_stream_t stream) {
+    if (!counts || !offsets) return MOE_ERR_NULL;
+    if (E <= 0) return MOE_ERR_SHAPE;
+    if (E > 1024) return MOE_ERR_LIMIT;
+    return launch_exclusive_scan_expert_offsets(counts, offsets, E, as_stream(stream));
+}
+
+int moe_compact_by_expert(const int* expert_ids, const int* tokens, const float* weights, int BK, const int* offsets,
+                          int* write_counters, int* tokens_flat, float* weights_flat, int E, moe_stream_t stream) {
+    if (!expert_ids || !tokens || !weights || !offsets || !write_counters || !tokens_flat || !weights_flat)
+        return MOE_ERR_NULL;
+    if (BK <= 0 || E <= 0) return MOE_ERR_SHAPE;
+    if (E > 1024 || BK >= (1 << 29)) return MOE_ERR_LIMIT;
+    return launch_compact_by_expert(expert_ids, tokens, weights, BK, offsets, write_counters, tokens_flat, weights_flat,
+                                    E, as_stream(stream));
+}
+
+int moe_classify_and_build_queues(const int* expert_offsets, int E, int very_sparse_cutoff, float heavy_factor_sparse,
+                                  float heavy_factor_default, int* wq_heavy, int* wq_light, moe_queue_stats* stats,
+                                  moe_stream_t stream) {
+    if (!expert_offsets || !wq_heavy || !wq_light || !stats) return MOE_ERR_NULL;
+    if (E <= 0) return MOE_ERR_SHAPE;
+    if (E > 1024) return MOE_ERR_LIMIT;
+    return launch_classify_and_build_queues(expert_offsets, E, very_sparse_cutoff, heavy_factor_sparse,
+                                            heavy_factor_default, wq_heavy, wq_light, stats, as_stream(stream));
+}
+
 int moe_build_work_queue(const int* expert_offsets, int E, int* work_queue, int* work_count, moe_stream_t stream) {
     if (!expert_offsets || !work_queue || !work_count) return MOE_ERR_NULL;
     if (E <= 0) return MOE_ERR_SHAPE;

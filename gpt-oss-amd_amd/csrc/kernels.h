@@ -4,6 +4,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+struct moe_queue_stats;  // include/moe_abi.h
+
 namespace moe {
 
 // ---- router.hip -------------------------------------------------------------------------------
@@ -49,6 +51,16 @@ int launch_gather_rows(const float* X, const int* idx, float* Y, int rows, int H
 int launch_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, hipStream_t stream);
 int launch_build_work_queue(const int* expert_offsets, int E, int* work_queue, int* work_count,
                             hipStream_t stream);
+
+// ---- scheduler_ref.hip: the reference's bucketing steps under their own argument lists ------------
+int launch_count_tokens_per_expert(const int* topk_i, const float* topk_v, int B, int K, int* out_expert,
+                                   int* out_token, float* out_w, int* counts, int E, hipStream_t stream);
+int launch_exclusive_scan_expert_offsets(int* counts, int* offsets, int E, hipStream_t stream);
+int launch_compact_by_expert(const int* expert_ids, const int* tokens, const float* weights, int BK, const int* offsets,
+                             int* write_counters, int* tokens_flat, float* weights_flat, int E, hipStream_t stream);
+int launch_classify_and_build_queues(const int* expert_offsets, int E, int very_sparse_cutoff,
+                                     float heavy_factor_sparse, float heavy_factor_default, int* wq_heavy,
+                                     int* wq_light, ::moe_queue_stats* stats, hipStream_t stream);
 
 // ---- experts_stream.hip ------------------------------------------------------------------------
 struct ExpertGemmArgs {

@@ -55,6 +55,31 @@ inline int bucket_by_expert(const int* topk_i, const float* topk_v, int B, int K
     return moe_bucket_by_expert(topk_i, topk_v, B, K, E, expert_offsets, tokens_flat, weights_flat, nullptr, stream);
 }
 
+// The same three steps one by one, under the kernels' own names and argument lists + the stream
+// (src/hip/scheduler.hip:11, 33, 48): `k<<<grid, block, 0, s>>>(args)` becomes `k(args, s)`;
+// compact_by_expert_kernel also takes the number of experts.
+using MoEStats = moe_queue_stats;  // src/hip/scheduler.hip:3-9
+inline int count_tokens_per_expert(const int* topk_i, const float* topk_v, int B, int K, int* out_expert,
+                                   int* out_token, float* out_w, int* counts, int E, moe_stream_t stream = nullptr) {
+    return moe_count_tokens_per_expert(topk_i, topk_v, B, K, out_expert, out_token, out_w, counts, E, stream);
+}
+inline int exclusive_scan_expert_offsets(int* counts, int* offsets, int E, moe_stream_t stream = nullptr) {
+    return moe_exclusive_scan_expert_offsets(counts, offsets, E, stream);
+}
+inline int compact_by_expert_kernel(const int* expert_ids, const int* tokens, const float* weights, int BK,
+                                    const int* offsets, int* write_counters, int* tokens_flat, float* weights_flat,
+                                    int E, moe_stream_t stream = nullptr) {
+    return moe_compact_by_expert(expert_ids, tokens, weights, BK, offsets, write_counters, tokens_flat, weights_flat, E,
+                                 stream);
+}
+// src/hip/scheduler.hip:112-119
+inline int classify_and_build_queues(const int* expert_offsets, int E, int very_sparse_cutoff,
+                                     float heavy_factor_sparse, float heavy_factor_default, int* wq_heavy,
+                                     int* wq_light, MoEStats* stats_out, moe_stream_t stream = nullptr) {
+    return moe_classify_and_build_queues(expert_offsets, E, very_sparse_cutoff, heavy_factor_sparse,
+                                         heavy_factor_default, wq_heavy, wq_light, stats_out, stream);
+}
+
 // src/hip/scheduler.hip:63-85, launched at src/forward.cpp:351-363
 inline int gather_rows(const float* X, const int* idx, float* Y, int BK, int H, moe_stream_t stream = nullptr) {
     return moe_gather_rows(X, idx, Y, BK, H, stream);

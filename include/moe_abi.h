@@ -150,6 +150,43 @@ MOE_API int moe_gather_rows(const float* X, const int* idx, float* Y, int rows, 
  * host/moe_getp.hpp keeps one state row per sequence instead and returns a step's rows with this. */
 MOE_API int moe_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, moe_stream_t stream);
 
+/* The reference's bucketing steps one by one, each under the argument list of the kernel it replaces
+ * plus the stream (the reference launches them inline with <<<grid, block, 0, stream>>>,
+ * src/forward.cpp:333-376), for a host loop that keeps those call sites.  moe_bucket_by_expert above
+ * does the first three in one launch.
+ *
+ * moe_count_tokens_per_expert: count_tokens_per_expert (src/hip/scheduler.hip:11-31).
+ *   out_expert / out_token / out_w [B*K] = the assignments (b, k) flattened in b-major order: expert id,
+ *   token b, routing weight; counts[e] += number of assignments to e (ids outside [0, E) are flattened
+ *   but not counted).  counts must be zero on entry, as in the reference.
+ * moe_exclusive_scan_expert_offsets: exclusive_scan_expert_offsets (:33-46).
+ *   offsets[0] = 0, offsets[i+1] = counts[0] + .. + counts[i]; counts is zeroed.
+ * moe_compact_by_expert: compact_by_expert_kernel (:48-61).
+ *   tokens_flat / weights_flat [BK] = tokens / weights grouped by expert at offsets[e]; write_counters[e]
+ *   grows by the bucket's size (zero on entry, as left by the scan).  Inside a bucket the entries keep
+ *   ascending assignment index; the reference's order there is the order its atomic slot claims
+ *   happen to finish.  One argument more than the reference kernel: E, the number of experts (the
+ *   grid is one block per expert).  Every id must be in [0, E).
+ * moe_classify_and_build_queues: classify_and_build_queues (:112-184), same decision rule, queues
+ *   and statistics; moe_queue_stats is its MoEStats (:3-9).  wq_heavy / wq_light hold up to 3*E ints.
+ * E <= 1024, B*K < 2^29. */
+typedef struct moe_queue_stats {
+    int heavy_count;
+    int light_count;
+    int heavy_maxNe;
+    int active_experts;
+    long long sumNe;
+} moe_queue_stats;
+MOE_API int moe_count_tokens_per_expert(const int* topk_i, const float* topk_v, int B, int K, int* out_expert,
+                                int* out_token, float* out_w, int* counts, int E, moe_stream_t stream);
+MOE_API int moe_exclusive_scan_expert_offsets(int* counts, int* offsets, int E, moe_stream_t stream);
+MOE_API int moe_compact_by_expert(const int* expert_ids, const int* tokens, const float* weights, int BK,
+                          const int* offsets, int* write_counters, int* tokens_flat, float* weights_flat, int E,
+                          moe_stream_t stream);
+MOE_API int moe_classify_and_build_queues(const int* expert_offsets, int E, int very_sparse_cutoff,
+                                  float heavy_factor_sparse, float heavy_factor_default, int* wq_heavy,
+                                  int* wq_light, moe_queue_stats* stats, moe_stream_t stream);
+
 /* Replaces classify_and_build_queues (src/hip/scheduler.hip:112-184; call site
  * src/forward.cpp:373-376).  One queue of (expert, row_offset, row_count) triples for the
  * non-empty experts in ascending expert id; work_count[0] receives their number.  The

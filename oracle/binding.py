@@ -27,8 +27,7 @@ def build(force=False):
 
 
 def _load():
-    if not os.path.exists(LIB_PATH):
-        build()
+    build()  # compiles when the library is missing or older than its source
     lib = ctypes.CDLL(LIB_PATH)
     sig = {
         "oracle_max_threads": (_i, []),
@@ -45,6 +44,7 @@ def _load():
         "oracle_bf16_to_f32": (None, [_vp, _ll, _vp]),
         "oracle_f32_to_bf16": (None, [_vp, _ll, _vp]),
         "oracle_bucket": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
+        "oracle_classify_queues": (None, [_vp, _i, _i, _f, _f, _vp, _vp, _vp]),
         "oracle_synth_normal_table": (None, [_vp]),
         "oracle_synth_normal_f32": (None, [_vp, _ll, _vp, _f, _u, _u, _ll]),
         "oracle_synth_normal_bf16": (None, [_vp, _ll, _vp, _f, _u, _u, _ll]),
@@ -191,6 +191,19 @@ def bucket(topk_i, topk_v, E):
     if rc:
         raise ValueError("oracle_bucket rc=%d" % rc)
     return offsets, tokens_flat, weights_flat, slot_of.reshape(T, K)
+
+
+def classify_queues(expert_offsets, very_sparse_cutoff, heavy_factor_sparse, heavy_factor_default):
+    """(wq_heavy [n_heavy, 3], wq_light [n_light, 3], stats) with stats = (heavy_count, light_count,
+    heavy_maxNe, active_experts, sumNe)."""
+    off = np.ascontiguousarray(expert_offsets, dtype=np.int32)
+    E = len(off) - 1
+    wq_h = np.full(3 * E, -1, dtype=np.int32)
+    wq_l = np.full(3 * E, -1, dtype=np.int32)
+    stats = np.zeros(5, dtype=np.int64)
+    _lib.oracle_classify_queues(_p(off), E, very_sparse_cutoff, heavy_factor_sparse, heavy_factor_default, _p(wq_h),
+                                _p(wq_l), _p(stats))
+    return wq_h[: 3 * stats[0]].reshape(-1, 3), wq_l[: 3 * stats[1]].reshape(-1, 3), tuple(int(v) for v in stats)
 
 
 # ---- synthetic inputs (include/moe_synth.h), host side ------------------------------------------

@@ -28,6 +28,10 @@
  *                                              reference claims slots with atomics, so order
  *                                              inside a bucket is unspecified there; here it
  *                                              is ascending token id
+ *   oracle_classify_queues src/hip/scheduler.hip:112-184  heavy / light work queues: experts with
+ *                                              rows, in ascending id, heavy when at most
+ *                                              `very_sparse_cutoff` experts are active or when the
+ *                                              expert has at least ceil(factor * mean rows) rows
  *
  * Pinning status (what fixes each function independently of this file):
  *   matmul/moe_block  : fp64 numpy composition, one-hot and zero inputs, brute force (tests)
@@ -37,6 +41,8 @@
  *   dequant           : exhaustive 16 codes x 256 scales against exact rational arithmetic and
  *                       against torch.ldexp on bf16 (the library routine the reference calls)
  *   bucket            : integer invariants (bincount, exclusive scan, sortedness, round trip)
+ *   classify_queues   : numpy restatement of the rule from its description (partition of the active
+ *                       experts, threshold cases at each of the three factor regimes, empty input)
  * The reference holds no golden vectors for this path and its translation unit does not
  * compile as shipped, so nothing here is checked against a reference binary.
  * PARITY UNPINNED (outside every workload's range): the NaN payload that scale byte 255
@@ -354,6 +360,56 @@ ORACLE_API int oracle_bucket(const int* topk_i, const float* topk_v, int T, int 
     }
     free(counts);
     return 0;
+}
+
+/* ---- src/hip/scheduler.hip:112-184 --------------------------------------------------- *
+ * expert_offsets [E+1] -> wq_heavy / wq_light (triples expert, row_offset, row_count, ascending
+ * expert id) and stats = {heavy_count, light_count, heavy_maxNe, active_experts, sumNe}.
+ */
+ORACLE_API void oracle_classify_queues(const int* expert_offsets, int E, int very_sparse_cutoff,
+                                       float heavy_factor_sparse, float heavy_factor_default,
+                                       int* wq_heavy, int* wq_light, long long* stats) {
+    int active = 0;
+    long long sum = 0;
+    for (int e = 0; e < E; ++e) {
+        int ne = expert_offsets[e + 1] - expert_offsets[e];
+        if (ne > 0) {
+            ++active;
+            sum += ne;
+        }
+    }
+    stats[0] = stats[1] = stats[2] = stats[3] = stats[4] = 0;
+    if (active == 0) return;
+    float avg = (float)sum / (float)active;
+    float factor = heavy_factor_default;
+    if (active <= very_sparse_cutoff)
+        factor = 1.0f;
+    else if (active <= 12)
+        factor = heavy_factor_sparse;
+    int thresh = (int)ceilf(factor * avg);
+    int nh = 0, nl = 0, hmax = 0;
+    for (int e = 0; e < E; ++e) {
+        int off = expert_offsets[e];
+        int ne = expert_offsets[e + 1] - off;
+        if (ne <= 0) continue;
+        if (active <= very_sparse_cutoff || ne >= thresh) {
+            wq_heavy[3 * nh + 0] = e;
+            wq_heavy[3 * nh + 1] = off;
+            wq_heavy[3 * nh + 2] = ne;
+            ++nh;
+            if (ne > hmax) hmax = ne;
+        } else {
+            wq_light[3 * nl + 0] = e;
+            wq_light[3 * nl + 1] = off;
+            wq_light[3 * nl + 2] = ne;
+            ++nl;
+        }
+    }
+    stats[0] = nh;
+    stats[1] = nl;
+    stats[2] = hmax;
+    stats[3] = active;
+    stats[4] = sum;
 }
 
 /* ---- synthetic inputs (include/moe_synth.h), host side -------------------------------- */

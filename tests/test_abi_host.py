@@ -61,6 +61,11 @@ def test_entries_reject_bad_arguments_without_a_device(pkg):
     assert L.moe_gemm_router(16, 8, 16, 16, 4, 2880, 32, 16, 1 << 30, None) == -6
     assert L.moe_bucket_by_expert(1, 1, 4, 4, 2000, 1, 1, 1, None, None) == -3
     assert L.moe_gather_rows(1, 1, 1, 4, 6, None) == -2
+    assert L.moe_count_tokens_per_expert(1, 1, 4, 4, 1, 1, 1, None, 32, None) == -1
+    assert L.moe_count_tokens_per_expert(1, 1, 4, 4, 1, 1, 1, 1, 2000, None) == -3
+    assert L.moe_exclusive_scan_expert_offsets(1, 1, 0, None) == -2
+    assert L.moe_compact_by_expert(1, 1, 1, 16, 1, 1, 1, None, 32, None) == -1
+    assert L.moe_classify_and_build_queues(1, 32, 6, 1.5, 1.25, 1, 1, None, None) == -1
     assert L.moe_dequant_mxfp4(8, 8, 4, 8, None) == -6      # blocks not 16-byte aligned
     assert L.moe_mxfp4_repack(16, 16, 1, 63, 64, 16, 16, None) == -2
     assert L.moe_block_forward(None, None) == -1

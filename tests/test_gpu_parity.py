@@ -165,6 +165,46 @@ def test_bucketing_bit_exact(pkg, oracle, dev, T, K, E):
     assert np.array_equal(q[:, 0], active) and np.array_equal(q[:, 1], r_off[active]) and np.array_equal(q[:, 2], counts[active])
 
 
+@pytest.mark.parametrize("T,K,E", [(1, 1, 1), (5, 2, 4), (256, 4, 32), (1024, 4, 128), (4100, 4, 32), (777, 8, 200)])
+def test_reference_signature_bucketing_steps(pkg, oracle, dev, T, K, E):
+    """count -> scan -> compact -> classify under the reference kernels' argument lists
+    (src/hip/scheduler.hip:11, 33, 48, 112) against the oracle, bit for bit."""
+    rng = np.random.default_rng(3 * T + E)
+    p = 1.0 / np.arange(1, E + 1) ** 1.2
+    p /= p.sum()
+    topk_i = np.stack([rng.choice(E, size=K, replace=False, p=p) for _ in range(T)]).astype(np.int32)
+    topk_v = rng.random((T, K)).astype(np.float32)
+    A = T * K
+    i32 = lambda n, v=0: torch.full((n,), v, dtype=torch.int32, device=dev)
+    a_e, a_t, counts, off = i32(A, -1), i32(A, -1), i32(E), i32(E + 1, -1)
+    a_w = torch.zeros(A, dtype=torch.float32, device=dev)
+    d_i, d_v = to_dev(topk_i, dev), to_dev(topk_v, dev)
+    pkg.count_tokens_per_expert(d_i, d_v, T, K, a_e, a_t, a_w, counts, E)
+    assert np.array_equal(a_e.cpu().numpy(), topk_i.ravel())
+    assert np.array_equal(a_t.cpu().numpy(), np.repeat(np.arange(T), K))
+    assert np.array_equal(a_w.cpu().numpy(), topk_v.ravel())
+    assert np.array_equal(counts.cpu().numpy(), np.bincount(topk_i.ravel(), minlength=E))
+    pkg.exclusive_scan_expert_offsets(counts, off, E)
+    r_off, r_tok, r_wts, _ = oracle.bucket(topk_i, topk_v, E)
+    assert np.array_equal(off.cpu().numpy(), r_off)
+    assert not counts.cpu().numpy().any()
+    tok, wts = i32(A, -1), torch.zeros(A, dtype=torch.float32, device=dev)
+    pkg.compact_by_expert(a_e, a_t, a_w, A, off, counts, tok, wts, E)
+    assert np.array_equal(tok.cpu().numpy(), r_tok)
+    assert np.array_equal(wts.cpu().numpy(), r_wts)
+    assert np.array_equal(counts.cpu().numpy(), np.diff(r_off))      # as after the reference's slot claims
+    for cutoff, fs, fd in [(6, 1.5, 1.25), (0, 2.0, 1.0)]:           # the reference's constants (src/forward.cpp:36-44) first
+        wq_h, wq_l = i32(3 * E, -1), i32(3 * E, -1)
+        stats = torch.zeros(3, dtype=torch.int64, device=dev)
+        pkg.classify_and_build_queues(off, E, cutoff, fs, fd, wq_h, wq_l, stats)
+        r_h, r_l, r_st = oracle.classify_queues(r_off, cutoff, fs, fd)
+        st32 = stats.cpu().numpy().view(np.int32)
+        got = (int(st32[0]), int(st32[1]), int(st32[2]), int(st32[3]), int(stats.cpu().numpy()[2]))
+        assert got == r_st
+        assert np.array_equal(wq_h.cpu().numpy()[: 3 * r_st[0]].reshape(-1, 3), r_h)
+        assert np.array_equal(wq_l.cpu().numpy()[: 3 * r_st[1]].reshape(-1, 3), r_l)
+
+
 # ---- whole block, small shapes (oracle on every token) ---------------------------------------------
 SMALL = [
     # T, H, I, E, K, fmt

@@ -228,6 +228,48 @@ def test_bucket_empty_experts_and_skew(oracle):
     assert tok.tolist() == list(range(10)) * 2
 
 
+# ---- heavy / light work queues: src/hip/scheduler.hip:112-184 -------------------------------------
+def numpy_classify(off, cutoff, f_sparse, f_default):
+    """The rule from its description, with library calls only: active experts split by a row threshold."""
+    ne = np.diff(off)
+    act = np.nonzero(ne > 0)[0]
+    if len(act) == 0:
+        return np.zeros((0, 3), np.int32), np.zeros((0, 3), np.int32), (0, 0, 0, 0, 0)
+    avg = np.float32(ne[act].sum()) / np.float32(len(act))
+    factor = np.float32(1.0 if len(act) <= cutoff else f_sparse if len(act) <= 12 else f_default)
+    thresh = int(np.ceil(np.float32(factor * avg)))
+    heavy = act if len(act) <= cutoff else act[ne[act] >= thresh]
+    light = np.setdiff1d(act, heavy)
+    q = lambda sel: np.stack([sel, off[sel], ne[sel]], axis=1).astype(np.int32).reshape(-1, 3)
+    return q(heavy), q(light), (len(heavy), len(light), int(ne[heavy].max()) if len(heavy) else 0, len(act), int(ne.sum()))
+
+
+def test_classify_queues_against_numpy(oracle):
+    rng = np.random.default_rng(12)
+    cases = [np.zeros(9, np.int64)]                                   # no rows at all
+    cases.append(np.concatenate([[0], np.cumsum([5, 0, 0, 7, 0, 1])]))  # 3 active <= cutoff 6: all heavy
+    cases.append(np.concatenate([[0], np.cumsum([10, 10, 10, 10, 10, 10, 10, 15, 14, 0])]))  # 9 active: sparse factor 1.5
+    for E in (13, 32, 128, 200):
+        for _ in range(4):
+            counts = rng.integers(0, 40, size=E) * (rng.random(E) < rng.choice([0.2, 0.6, 1.0]))
+            cases.append(np.concatenate([[0], np.cumsum(counts)]))
+    # a bucket exactly at the threshold and one row below it (13 active experts, default factor 1.25)
+    counts = np.array([8] * 11 + [10, 9])        # mean 8.2308, 1.25 * mean = 10.29 -> threshold 11
+    cases.append(np.concatenate([[0], np.cumsum(counts)]))
+    counts = np.array([8] * 11 + [12, 4])        # mean 8 -> threshold exactly 10
+    cases.append(np.concatenate([[0], np.cumsum(counts)]))
+    for off in cases:
+        off = np.asarray(off, dtype=np.int32)
+        for cutoff, fs, fd in [(6, 1.5, 1.25), (0, 2.0, 1.0), (3, 1.0, 3.0)]:
+            h, l, st = oracle.classify_queues(off, cutoff, fs, fd)
+            rh, rl, rst = numpy_classify(off, cutoff, fs, fd)
+            assert np.array_equal(h, rh) and np.array_equal(l, rl) and st == rst, (off.tolist(), cutoff, fs, fd)
+            # partition of the active experts, ascending inside each queue
+            both = np.concatenate([h[:, 0], l[:, 0]])
+            assert np.array_equal(np.sort(both), np.nonzero(np.diff(off) > 0)[0])
+            assert np.all(np.diff(h[:, 0]) > 0) and np.all(np.diff(l[:, 0]) > 0)
+
+
 # ---- whole block: src/run.cpp:628-707 ------------------------------------------------------------
 def fp64_block(t, wr, br, w1, b1, w2, b2, K, limit=7.0):
     """Independent composition in numpy fp64 (library matmul, library sort)."""
