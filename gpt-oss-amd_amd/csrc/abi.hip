@@ -27,14 +27,13 @@ constexpr int kPrefillTileTokens = 128;
 // Which family runs the expert GEMMs, by average bucket size T*K/E (measured crossovers, 20b
 // shapes, token counts 256..4096).  MXFP4: the 128-token-block kernels win as soon as buckets start
 // to overflow one 64-token block (the streaming kernel then reads an expert's weights once per
-// block of its bucket).  bf16: the streaming kernel stays ahead up to a few hundred rows per expert
-// (the second block of a bucket finds the weights in the Infinity Cache, and the 128-token bf16
-// kernel has no direct-to-LDS staging).
+// block of its bucket).  bf16: the same (E = 32: 350 against 428 us at 48 rows per expert, 572 against
+// 437 us at 64).
 inline bool use_prefill_kernels(int T, int K, int E, int format, unsigned flags) {
     if (flags & MOE_FLAG_FORCE_STREAM) return false;
     if (flags & MOE_FLAG_FORCE_TILED) return true;
     const long long rows = (long long)T * K;
-    return format == MOE_WEIGHTS_MXFP4_TILED ? rows >= 52LL * E : rows >= 448LL * E;
+    return format == MOE_WEIGHTS_MXFP4_TILED ? rows >= 52LL * E : rows >= 56LL * E;
 }
 
 // Bucketing inside the expert kernels instead of a launch of its own: for the weight-streaming
@@ -465,7 +464,10 @@ struct ExpertPlan {
     // 32 rows each.  Blocks run in rounds of one per CU, so the cheaper choice is the one with the
     // smaller rounds x rows-per-block product; more rows per block also re-read the activations less.
     int pick_kernel(int rows) const {
-        if (prefill) return 16;
+        if (prefill) {  // bf16 weights, buckets of 80 rows and more on average: the one-block-a-CU kernel
+            const bool big = (long long)p->n_tokens * p->experts_per_token >= 80LL * p->n_experts;
+            return p->weight_format == MOE_WEIGHTS_BF16 && big ? 17 : 16;
+        }
         const int cost10 = ceil_div(ceil_div(rows / 32, 10) * est_tiles, n_cus) * 10;
         const int cost12 = ceil_div(ceil_div(rows / 32, 12) * est_tiles, n_cus) * 12;
         return cost12 <= cost10 ? 1 : 0;
@@ -685,7 +687,9 @@ int moe_block_describe(const moe_block_params* p, char* text, size_t text_bytes)
         int kernel = plan.pick_kernel(rows), row_blocks = plan.pick_row_blocks(rows, kernel);
         if (direct && fmt == MOE_WEIGHTS_MXFP4_TILED) plan.pick_two_pass(rows, &kernel, &row_blocks);
         const int cons = kernel == 1 ? 12 : 10;
-        if (prefill) {
+        if (prefill && kernel == 17) {
+            snprintf(out, n, "expert_prefill_bf16_kernel<%d>", epi);
+        } else if (prefill) {
             snprintf(out, n, "expert_prefill_kernel<%d, %d, 4>", fmt, epi);
         } else if (direct) {
             // as the launcher: at least enough row blocks for one (bf16) or two (MXFP4) passes of `cons` row units

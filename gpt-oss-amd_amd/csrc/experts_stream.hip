@@ -420,6 +420,15 @@ MOE_DEVICE void dma16(const void* gsrc, uint8_t* lds_dst_wave_uniform) {
                                      (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 16, 0, 0);
 }
 
+// The same load in assembly, the LDS address given as a wave-uniform integer (held in a scalar register
+// by the caller), for a wave that issues these loads several stages ahead and also reads LDS fragments
+// itself: the compiler puts a wait for every direct-to-LDS load it knows of in front of the wave's next
+// LDS read, so a ring of such loads must be invisible to it.  The load does count in vmcnt; the caller
+// waits for it itself.  Writes M0: a kernel that uses this must not use the builtin form as well.
+MOE_DEVICE void dma16_asm(const void* gsrc, uint32_t lds_addr_uniform) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gsrc), "s"(lds_addr_uniform)
+                 : "memory");
+}
 
 // LDS image of one stage of activations: token tile t at t*4096, row q (0..15) of the tile at
 // q*256, and inside the row the sixteen 16-byte chunks of the stage's 128 contraction elements,
@@ -1312,6 +1321,193 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     stream_epilogue<R, NT, EPI>(a, acc, e, [&](int i) { return row0 + i; }, nrows, unit, 0, bias_raw);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Prefill-sized buckets, bf16 weights.  A 128-token block needs its expert's rows from HBM (2 bytes a
+// weight, 128 flops a byte: the launch is bound by that stream), so everything here serves keeping
+// loads far ahead: ONE block of four waves per CU, i.e. one wave per SIMD with the whole register file
+// (128 accumulator registers for the 64 x 128 tile + a ring of three stages of weight registers, 192, so
+// weights are requested two stages = 256 contraction elements ahead) and 96 KiB of LDS (a ring of
+// three 128-token activation stages, moved global -> LDS two stages ahead by direct-to-LDS loads).
+// Order of issue in stage s: the weights of stage s + 2 (ordinary loads), the first MFMA group of stage
+// s (in front of which the compiler puts its wait for the weights of s: it knows of the 32 ordinary
+// loads issued since and not of the direct-to-LDS loads between them, so its wait also covers the
+// activations of stage s + 1), then the direct-to-LDS loads of stage s + 2 in assembly.  The stage
+// ends with an explicit wait for the activations of stage s + 1 (everything but the 16 + NT loads
+// issued after them) and the barrier.  The one or two stages after the last whole turn of the ring
+// request nothing and wait for every load: a count of younger loads holds only where those loads are
+// in the code, and the compiler removes weight loads whose registers no later stage reads.  Weight elements of k-step j (0..3) and lane group g: 64 (j/2) + 16 g + 8 (j%2)
+// .. +8, as in the producer/consumer kernel (a lane's two loads of a pair of steps are adjacent).
+// ---------------------------------------------------------------------------------------------
+constexpr int kBf16PrefillRing = 3;
+
+template <int NT, int EPI>
+MOE_DEVICE void prefill_body_bf16(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit,
+                                  bool active) {
+    constexpr int R = 4;
+    constexpr int D = kBf16PrefillRing;
+    constexpr int kSlotBytes = kStageSteps * 8 * 1024;  // 128 tokens x 128 elements x 2 bytes
+    constexpr int kYounger = (D - 2) * (4 * R + NT);    // loads of the stages requested after the next one
+    static_assert(kYounger <= 63, "vmcnt holds six bits");
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane & 15;
+    const int g = lane >> 4;
+    const int K = a.K;
+    const int n_stages = ceil_div(K, kStageElems);
+
+    // activation staging: this wave moves the four-row block `wave` of every token tile, 256 contiguous
+    // bytes per row (chunk c of row q stored at position c ^ q)
+    const int q_dma = 4 * wave + (lane >> 4);
+    const int chunk_dma = (lane & 15) ^ q_dma;
+    const uint8_t* b_row[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+        const int idx = min(i * 16 + q_dma, nrows - 1);
+        const int src = a.gather ? a.tokens_flat[row0 + idx] : row0 + idx;
+        b_row[i] = reinterpret_cast<const uint8_t*>(a.act + (size_t)src * K);
+    }
+    const uint32_t lds_dma0 = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(lds + wave * 1024));
+    auto issue_b = [&](int s) {
+        const int k = s * kStageElems + 8 * chunk_dma;
+        const size_t off = (k < K) ? (size_t)k * 2 : 0;  // past the row (or the last stage): re-read its start
+        const uint32_t dst = lds_dma0 + (uint32_t)(s % D) * kSlotBytes;
+#pragma unroll
+        for (int i = 0; i < NT; ++i) dma16_asm(b_row[i] + off, dst + i * 4096);
+    };
+    const uint8_t* const lds_rd = lds + (size_t)q * 256;
+    // slot: ring slot of the stage (compile-time in the stage code)
+    auto b_frag = [&](int slot, int j, int t) {
+        return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)slot * kSlotBytes + t * 4096 +
+                                               ((ws_chunk<FMT_BF16>(j, g) ^ q) << 4));
+    };
+
+    if (!active) {  // no row unit: this wave only moves its share of the activations
+#pragma unroll
+        for (int s = 0; s < D - 1; ++s) issue_b(s);
+        wait_vmcnt<(D - 2) * NT>();
+        __syncthreads();
+        for (int s = 0; s < n_stages; ++s) {
+            if (s < D * (n_stages / D)) {  // as the waves with rows: the stages of whole ring turns request
+                issue_b(s + D - 1);
+                wait_vmcnt<(D - 2) * NT>();
+            } else {
+                wait_vmcnt<0>();
+            }
+            __syncthreads();
+        }
+        wait_vmcnt<0>();  // nothing may still be writing this block's LDS when the wave ends
+        return;
+    }
+
+    const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
+    const uint8_t* a_ptr[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)(unit * 64 + tile_row_in_group(r, q)) * K);
+    // byte offset inside a row of this lane's eight elements of k-step j at stage 0
+    const int k_lane0 = 16 * g;
+    f32x4 acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    u32x4 araw[D][kStageSteps][R];
+    auto load_a = [&](int slot, int s) {
+#pragma unroll
+        for (int j = 0; j < kStageSteps; ++j) {
+            const int k = s * kStageElems + 64 * (j >> 1) + k_lane0 + 8 * (j & 1);
+            const size_t off = (k < K) ? (size_t)k * 2 : 0;  // past the row: re-read its start (zeroed at use)
+#pragma unroll
+            for (int r = 0; r < R; ++r) araw[slot][j][r] = *reinterpret_cast<const u32x4*>(a_ptr[r] + off);
+        }
+    };
+    // stage s in ring slot i (compile-time).  AHEAD: the loop's stages request stage s + 2; the last
+    // stages, after the loop, request nothing and wait for everything (a count of younger loads is only
+    // right where those loads are certain to be in the code: the compiler drops loads whose registers
+    // no later stage reads).
+    auto do_stage = [&](auto i_tag, auto ahead_tag, int s) {
+        constexpr int i = decltype(i_tag)::value;
+        constexpr bool AHEAD = decltype(ahead_tag)::value;
+        if constexpr (AHEAD) load_a((i + D - 1) % D, s + D - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 bq[2];
+        bq[0] = b_frag(i, 0, 0);
+        bq[1] = b_frag(i, 0, 1);
+#pragma unroll
+        for (int j = 0; j < kStageSteps; ++j) {
+            // elements past the contraction length (ragged last stage) multiply as zeros
+            const bool live = s * kStageElems + 64 * (j >> 1) + k_lane0 + 8 * (j & 1) < K;
+            u32x4 av[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) av[r] = live ? araw[i][j][r] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const u32x4 b = bq[t & 1];
+                if (t + 2 < NT) bq[t & 1] = b_frag(i, j, t + 2);
+                else if (j + 1 < kStageSteps) bq[t & 1] = b_frag(i, j + 1, t + 2 - NT);
+                __builtin_amdgcn_sched_barrier(0);  // keep the read above ahead of the MFMAs below
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r][t] = mfma_16x16x32(av[r], b, acc[r][t]);
+                if (AHEAD && j == 0 && t == 0) {
+                    __builtin_amdgcn_sched_barrier(0);  // this stage's weights have been waited for: now the
+                    issue_b(s + D - 1);                 // direct-to-LDS loads two stages ahead
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        wait_vmcnt<AHEAD ? kYounger : 0>();  // the activations of stage s + 1 have landed (and everything older)
+        __syncthreads();
+    };
+    uint2 bias_raw[R];
+    load_bias<R>(a, e, unit, 0, bias_raw);
+    static_assert(D == 3, "the stage loop below walks the ring in threes");
+    load_a(0, 0);
+    issue_b(0);
+    load_a(1, 1);
+    issue_b(1);
+    wait_vmcnt<kYounger>();  // stage 0's activations
+    __syncthreads();
+    // whole turns of the ring in the loop (when nothing is left over, its last requests re-read the rows'
+    // starts into slots nobody reads again), then the one or two stages left over
+    const int full_turns = n_stages / D;
+    using std::integral_constant;
+    for (int tr = 0; tr < full_turns; ++tr) {
+        do_stage(integral_constant<int, 0>{}, std::true_type{}, D * tr + 0);
+        do_stage(integral_constant<int, 1>{}, std::true_type{}, D * tr + 1);
+        do_stage(integral_constant<int, 2>{}, std::true_type{}, D * tr + 2);
+    }
+    const int tail = n_stages - D * full_turns;  // block-uniform
+    if (tail > 0) do_stage(integral_constant<int, 0>{}, std::false_type{}, D * full_turns + 0);
+    if (tail > 1) do_stage(integral_constant<int, 1>{}, std::false_type{}, D * full_turns + 1);
+    wait_vmcnt<0>();  // nothing may still be writing this block's LDS when the wave ends
+    stream_epilogue<R, NT, EPI>(a, acc, e, [&](int i) { return row0 + i; }, nrows, unit, 0, bias_raw);
+}
+
+// One block of four waves per CU (one wave per SIMD: 512 registers a lane, 128 KiB of LDS).  Block
+// index -> (token block, row block) as in expert_prefill_kernel.
+template <int EPI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void expert_prefill_bf16_kernel(ExpertGemmArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kBf16PrefillRing * kStageSteps * 8 * 1024];
+    const int n_rb = a.row_blocks;
+    const int xcd = blockIdx.x & 7;
+    const int m = blockIdx.x >> 3;
+    const int tile = (m / n_rb) * 8 + xcd;
+    const int row_block = m % n_rb;
+    if (tile >= *a.n_tiles) return;  // block-uniform
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int unit = row_block * 4 + wave;
+    const bool active = unit < a.rows / 64;
+    const int e = a.tile_expert[tile];
+    const int row0 = a.tile_row0[tile];
+    const int nrows = a.tile_rows[tile];
+    const int nt = (nrows + 15) >> 4;  // block-uniform
+    if (nt > 6) prefill_body_bf16<8, EPI>(a, lds, e, row0, nrows, unit, active);
+    else if (nt > 4) prefill_body_bf16<6, EPI>(a, lds, e, row0, nrows, unit, active);
+    else if (nt > 2) prefill_body_bf16<4, EPI>(a, lds, e, row0, nrows, unit, active);
+    else prefill_body_bf16<2, EPI>(a, lds, e, row0, nrows, unit, active);
+}
+
 template <int FMT, int NT, int EPI, int WAVES>
 MOE_DEVICE void prefill_body(const ExpertGemmArgs& a, uint8_t* lds, int e, int row0, int nrows, int unit, bool active) {
     if constexpr (FMT == FMT_MXFP4) {
@@ -1392,10 +1588,16 @@ int launch_cfg(const ExpertGemmArgs& a, hipStream_t stream) {
             } else {
                 hipLaunchKernelGGL((expert_stream_direct_kernel<FMT, EPI, 10, 2, false>), grid, dim3(768), 0, stream, b);
             }
-        } else if (a.waves_per_block == 16) {
+        } else if (a.waves_per_block == 16 || a.waves_per_block == 17) {
             ExpertGemmArgs b = a;
             b.row_blocks = ceil_div(a.rows / 64, 4);
             dim3 grid(ceil_div(a.max_tiles, 8) * 8 * b.row_blocks);  // every XCD gets whole token blocks
+            if constexpr (FMT == FMT_BF16) {
+                if (a.waves_per_block == 17) {
+                    hipLaunchKernelGGL((expert_prefill_bf16_kernel<EPI>), grid, dim3(256), 0, stream, b);
+                    return launch_status();
+                }
+            }
             hipLaunchKernelGGL((expert_prefill_kernel<FMT, EPI, 4>), grid, dim3(256), 0, stream, b);
         } else if (a.waves_per_block == 0) {
             ExpertGemmArgs b = a;

@@ -97,7 +97,9 @@ struct ExpertGemmArgs {
     int xcd_tiles;              // producer-consumer kernel: all row blocks of a token block on one XCD
     int waves_per_block;        // kernel choice of the fused block: 0 / 1 producer-consumer kernel with 10 / 12
                                 // consumer waves (+ 2 producers), 64-token blocks; 16 prefill kernel (4 waves,
-                                // 128-token blocks).  Ignored by the work-queue entries.
+                                // 128-token blocks, two blocks a CU); 17 bf16 weights only: prefill kernel with
+                                // one block a CU and a register ring of weights (MXFP4: as 16).  Ignored by the
+                                // work-queue entries.
 };
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
 int expert_direct_max_assignments();

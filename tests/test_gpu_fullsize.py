@@ -109,6 +109,27 @@ def test_prefill4096_mxfp4_zipf(pkg, wl, oracle, dev):
     assert hostgen.rel_err(ys.cpu().numpy(), y.cpu().numpy()) <= 1e-5
 
 
+def test_prefill4096_bf16(pkg, wl, oracle, dev):
+    """4096 tokens on the bf16 experts of the 20b-shaped block (512 rows an expert on average: the
+    128-token-block kernel with one block a compute unit)."""
+    shape = wl.MoeShape("prefill4096_bf16", T=4096)
+    blk, raw, x, y, ti, tv = run_block(wl, oracle, dev, shape)
+    tokens = np.sort(np.random.default_rng(2).choice(shape.T, 160, replace=False))
+    check_tokens(wl, oracle, shape, x, y, ti, tv, tokens, hostgen.host_layer(oracle, wl, shape))
+    properties(pkg, blk, x, y, ti, tv, shape)
+    # the same tokens through the decode-sized kernels and through the 128-token-block kernel that
+    # runs two blocks a compute unit (what 1000 of these tokens alone would get) agree closely
+    ys, tis, _ = blk.forward(x, flags=pkg.MOE_FLAG_FORCE_STREAM)
+    assert torch.equal(tis, ti)
+    e_s = hostgen.rel_err(ys.cpu().numpy(), y.cpu().numpy())
+    y1, ti1, _ = blk.forward(x[:600].contiguous(), flags=pkg.MOE_FLAG_FORCE_TILED)
+    assert torch.equal(ti1, ti[:600])
+    e_1 = hostgen.rel_err(y1.cpu().numpy(), y[:600].cpu().numpy())
+    say("  against the 64-token-block kernels %.3e, against the two-blocks-a-unit kernel %.3e" % (e_s, e_1))
+    assert e_s <= 1e-5
+    assert e_1 <= 1e-3  # another summation order ahead of the bf16 rounding of the SwiGLU rows
+
+
 @pytest.mark.parametrize("fmt", ["bf16", "mxfp4"])
 def test_largest_batch(pkg, wl, oracle, dev, fmt):
     """The documented maximum of 65535 tokens per call (small H and I keep it cheap): every launch grid

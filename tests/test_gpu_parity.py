@@ -224,6 +224,11 @@ SMALL = [
     (700, 320, 192, 8, 4, "bf16"),
     (210, 256, 128, 4, 2, "mxfp4"),      # ~105 rows per expert: one partly filled 128-token block each
     (97, 576, 320, 2, 2, "mxfp4"),       # 97 rows per expert, rows not a multiple of 512
+    # bf16 buckets of 80+ rows (one-block-a-CU kernel): contraction lengths of 2 / 5 and 4 / 7 stages of 128,
+    # i.e. one or two stages left after the whole turns of its three-stage ring, many token blocks in flight
+    (700, 192, 64, 64, 8, "bf16"),
+    (400, 576, 448, 8, 2, "bf16"),
+    (97, 576, 832, 2, 2, "bf16"),
 ]
 
 
