@@ -439,6 +439,19 @@ template <int FMT>
 MOE_DEVICE int ws_chunk(int j, int g) {  // chunk holding the operand of MFMA step j for lane group g
     return (FMT == FMT_BF16) ? 8 * (j >> 1) + 2 * g + (j & 1) : 4 * g + j;
 }
+// MXFP4: the image is built over a permutation of the chunks.  The LDS serves a fragment read with the
+// four lane groups of a token row side by side, and the chunks 4g + j that they read in one MFMA step
+// are 64 bytes apart: two of the four would share banks (measured: every fragment read took twice its
+// cycles).  ws_pos(c) takes the place of c above: chunk 4g + j sits where the bf16 operand order has
+// its step-j chunk of group g (32 bytes apart: no conflicts).  ws_chunk_at is the inverse.
+template <int FMT>
+MOE_DEVICE int ws_pos(int c) {
+    return (FMT == FMT_BF16) ? c : 8 * ((c & 3) >> 1) + 2 * (c >> 2) + (c & 1);
+}
+template <int FMT>
+MOE_DEVICE int ws_chunk_at(int p) {
+    return (FMT == FMT_BF16) ? p : 4 * ((p >> 1) & 3) + (((p >> 3) << 1) | (p & 1));
+}
 
 // act_row(i): row of a.act that holds bucket row i of the token block (i < nrows).
 // The stages of the bucket's rows are streamed `passes` times over (once per pass of the consumers
@@ -463,7 +476,7 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row
 #pragma unroll
     for (int ii = 0; ii < BP; ++ii) {
         const int q = 4 * (BP * p + ii) + sub;
-        chunk[ii] = pos ^ q;
+        chunk[ii] = ws_chunk_at<FMT>(pos ^ q);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int idx = min(t * 16 + q, nrows - 1);
@@ -535,7 +548,7 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
     const uint8_t* const lds_rd = lds + (size_t)q * 256;
     auto b_frag = [&](int s, int j, int t) {
         return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & (kWsRing - 1)) * kLdsStageBytes + t * 4096 +
-                                               ((ws_chunk<FMT>(j, g) ^ q) << 4));
+                                               ((ws_pos<FMT>(ws_chunk<FMT>(j, g)) ^ q) << 4));
     };
     f32x4 acc[R][NT];
 #pragma unroll
@@ -726,7 +739,7 @@ MOE_DEVICE void ws_consumer_two(const ExpertGemmArgs& a, const uint8_t* lds, int
     // gs: stage counted over all passes (the producers' ring slot)
     auto b_frag = [&](int gs, int j, int t) {
         return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(gs & (kWsRing - 1)) * kLdsStageBytes + t * 4096 +
-                                               ((ws_chunk<FMT>(j, g) ^ q) << 4));
+                                               ((ws_pos<FMT>(ws_chunk<FMT>(j, g)) ^ q) << 4));
     };
     f32x4 acc[R][NT];
     uint2 bias_raw[R];
@@ -1199,7 +1212,7 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     const int blk_w = wave & 3;
     const int half_w = wave >> 2;
     const int q_dma = 4 * blk_w + (lane >> 4);     // row of the token tile this lane moves
-    const int chunk_dma = (lane & 15) ^ q_dma;     // chunk of the stage it fetches
+    const int chunk_dma = ws_chunk_at<FMT_MXFP4>((lane & 15) ^ q_dma);  // chunk of the stage it fetches
     const uint8_t* b_row[TS];
 #pragma unroll
     for (int i = 0; i < TS; ++i) {
@@ -1217,7 +1230,7 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
     const uint8_t* const lds_rd = lds + (size_t)q * 256;
     auto b_frag = [&](int s, int j, int t) {  // lane group g owns MX block g of a stage: chunk 4g + j
         return *reinterpret_cast<const u32x4*>(lds_rd + (size_t)(s & 1) * kStageBytes + t * 4096 +
-                                               (((4 * g + j) ^ q) << 4));
+                                               ((ws_pos<FMT_MXFP4>(4 * g + j) ^ q) << 4));
     };
 
     if (!active) {

@@ -44,6 +44,7 @@ WORKLOADS = {
     "decode256_bf16": MoeShape("decode256_bf16", T=256),
     "decode256_mxfp4": MoeShape("decode256_mxfp4", T=256, fmt="mxfp4"),
     "prefill4096_mxfp4_zipf": MoeShape("prefill4096_mxfp4_zipf", T=4096, fmt="mxfp4", zipf_s=1.2),
+    "prefill4096_bf16": MoeShape("prefill4096_bf16", T=4096),
     "layer120b_mxfp4": MoeShape("layer120b_mxfp4", T=1024, E=128, fmt="mxfp4"),
     "stack120b_mxfp4": MoeShape("stack120b_mxfp4", T=1024, E=128, fmt="mxfp4", layers=36),
 }

@@ -112,7 +112,7 @@ def test_prefill4096_mxfp4_zipf(pkg, wl, oracle, dev):
 def test_prefill4096_bf16(pkg, wl, oracle, dev):
     """4096 tokens on the bf16 experts of the 20b-shaped block (512 rows an expert on average: the
     128-token-block kernel with one block a compute unit)."""
-    shape = wl.MoeShape("prefill4096_bf16", T=4096)
+    shape = wl.WORKLOADS["prefill4096_bf16"]
     blk, raw, x, y, ti, tv = run_block(wl, oracle, dev, shape)
     tokens = np.sort(np.random.default_rng(2).choice(shape.T, 160, replace=False))
     check_tokens(wl, oracle, shape, x, y, ti, tv, tokens, hostgen.host_layer(oracle, wl, shape))
