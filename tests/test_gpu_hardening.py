@@ -38,7 +38,10 @@ def routing(T, E, K, seed):
 
 
 # T, H, I, E, K : I is the contraction length of the down GEMM (320 = ragged last MX stage; 2880 real)
-ONE_HOT = [(70, 128, 320, 8, 4), (33, 192, 2880, 4, 2), (300, 64, 320, 4, 4), (129, 2880, 2880, 8, 4)]
+# the last two: buckets of 100 / 200 rows (bf16: the 128-token-block kernel with one block a compute unit), whose
+# three-stage ring leaves two stages (2880 = 22.5 stages of 128) / one stage (448 = 3.5) after its whole turns
+ONE_HOT = [(70, 128, 320, 8, 4), (33, 192, 2880, 4, 2), (300, 64, 320, 4, 4), (129, 2880, 2880, 8, 4),
+           (400, 2880, 2880, 8, 2), (200, 64, 448, 2, 2)]
 
 
 @pytest.mark.parametrize("fmt", ["mxfp4", "bf16"])
