@@ -339,6 +339,43 @@ def test_block_random_shapes(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
         assert err <= OUT_TOL, (flags, err)
 
 
+def _random_bucket_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        E = int(rng.choice([2, 3, 4, 6, 8, 12]))
+        K = int(rng.integers(1, min(4, E) + 1))
+        T = int(rng.choice([90, 130, 200, 333, 512, 700, 1025, 1500]))
+        H = 64 * int(rng.integers(1, 13))
+        I = 64 * int(rng.integers(1, 13))
+        out.append((T, H, I, E, K, ["bf16", "mxfp4"][i % 2]))
+    return out
+
+
+@pytest.mark.parametrize("T,H,I,E,K,fmt", _random_bucket_shapes(20, seed=31))
+def test_block_random_long_buckets(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
+    """Seeded random shapes with few experts and up to 1500 tokens: buckets of tens to hundreds of rows
+    (several token blocks per expert, every 128-token-block kernel), contraction lengths of 1 to 6 stages
+    of 128 with and without a ragged last one; the size rule's choice and every forced family."""
+    shape = wl.MoeShape("randlong", T=T, H=H, I=I, E=E, K=K, fmt=fmt, seed=2000 + T + 3 * H + I + E)
+    say("block_random_long", shape, "rows per expert %.0f" % (T * K / E))
+    table = oracle.normal_table()
+    blk, raw = wl.make_device_layer(shape, table, dev)
+    x = wl.make_device_input(shape, table, dev)
+    hw = hostgen.host_layer(oracle, wl, shape)
+    ref_y, ref_i, ref_v, _ = hostgen.oracle_block(oracle, shape, hw, hostgen.host_input(oracle, wl, shape))
+    families = [0, pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH, pkg.MOE_FLAG_FORCE_TILED]
+    if T * K <= 4096:  # the longest assignment list a block scans itself
+        families.append(pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT)
+    for flags in families:
+        y, ti, tv = blk.forward(x, flags=flags)
+        torch.cuda.synchronize()
+        assert np.array_equal(ti.cpu().numpy(), ref_i), flags
+        np.testing.assert_allclose(tv.cpu().numpy(), ref_v, rtol=2e-6)
+        err = hostgen.rel_err(y.cpu().numpy(), ref_y)
+        assert err <= OUT_TOL, (flags, err)
+
+
 def test_block_residual_and_rmsnorm_glue(pkg, wl, oracle, dev):
     shape = wl.MoeShape("glue", T=40, H=256, I=128, E=8, K=4, fmt="bf16", seed=3)
     table = oracle.normal_table()
