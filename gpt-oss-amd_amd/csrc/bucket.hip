@@ -28,8 +28,8 @@ __global__ __launch_bounds__(1024) void bucket_kernel(const int* __restrict__ to
                                                       float* __restrict__ weights_flat,
                                                       int* __restrict__ slot_of, TileMap map) {
     extern __shared__ int lds[];
+    __shared__ int wave_cnt[4 * 16];  // matches per wave of the four compaction steps in flight
     int* hist = lds;                  // [E]
-    int* wave_cnt = lds + E;          // [16]
     int* scal = lds + E + 16;         // [0] rows before this expert, [1] full tiles before it, [2] full tiles in all,
                                       // [3] partial tiles ahead of this expert's (by size), [4] partial tiles in all,
                                       // [5] partial tiles of the experts before this one
@@ -143,31 +143,34 @@ __global__ __launch_bounds__(1024) void bucket_kernel(const int* __restrict__ to
             const int t = t00 + u * 1024 + tid;
             wv4[u] = mk4[u] >= 0 ? topk_v[(size_t)t * K + mk4[u]] : 0.f;
         }
+        // the four steps' wave counts go through LDS together: one exchange (two barriers) per 4096 tokens
+        int prefix4[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            if (t00 + u * 1024 >= T) break;  // block-uniform
+            const unsigned long long ballot = __ballot(mk4[u] >= 0);
+            prefix4[u] = __popcll(ballot & ((1ull << lane) - 1ull));
+            if (lane == 0) wave_cnt[u * 16 + wave] = __popcll(ballot);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
             const int t = t00 + u * 1024 + tid;
-            const int mk = mk4[u];
-            const unsigned long long ballot = __ballot(mk >= 0);
-            const int prefix = __popcll(ballot & ((1ull << lane) - 1ull));
-            if (lane == 0) wave_cnt[wave] = __popcll(ballot);
-            __syncthreads();
             int wave_base = 0, total = 0;
 #pragma unroll
             for (int w = 0; w < 16; ++w) {
-                const int c = wave_cnt[w];
+                const int c = wave_cnt[u * 16 + w];
                 if (w < wave) wave_base += c;
                 total += c;
             }
-            if (mk >= 0) {
-                const int dst = base + wave_base + prefix;
+            if (mk4[u] >= 0) {
+                const int dst = base + wave_base + prefix4[u];
                 tokens_flat[dst] = t;
                 weights_flat[dst] = wv4[u];
-                if (slot_of) slot_of[(size_t)t * K + mk] = dst;
+                if (slot_of) slot_of[(size_t)t * K + mk4[u]] = dst;
             }
             base += total;
-            __syncthreads();
         }
+        __syncthreads();
     }
 }
 
