@@ -63,3 +63,33 @@ def test_graph_replays_equal_the_eager_call(pkg, wl, oracle, dev, T, H, I, E, K,
         # eager work on the same buffers between the replays
         got = eager(inp)
         assert torch.equal(got[0], ref[0])
+
+
+def test_two_streams_do_not_share_state(pkg, wl, oracle, dev):
+    """Two calls with their own workspaces on two streams at once (default priority) give the bits each gives
+    alone: the library keeps nothing between or across calls."""
+    table = oracle.normal_table()
+    jobs = []
+    for T, H, I, E, K, fmt in ((256, 256, 128, 8, 4, "mxfp4"), (700, 320, 192, 8, 4, "bf16")):
+        shape = wl.MoeShape("streams", T=T, H=H, I=I, E=E, K=K, fmt=fmt, seed=T)
+        blk, raw = wl.make_device_layer(shape, table, dev)
+        x = wl.make_device_input(shape, table, dev)
+        out = (torch.empty((T, H), dtype=torch.float32, device=dev), torch.empty((T, K), dtype=torch.int32, device=dev),
+               torch.empty((T, K), dtype=torch.float32, device=dev))
+        p = blk.params(x, *out)
+        blk.launch(p, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        jobs.append((blk, raw, x, p, out, [o.clone() for o in out]))
+    streams = [torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)]
+    torch.cuda.synchronize()
+    for _ in range(20):
+        for (blk, raw, x, p, out, alone), st in zip(jobs, streams):
+            for o in out:
+                o.zero_()
+        torch.cuda.synchronize()
+        for _ in range(3):
+            for (blk, raw, x, p, out, alone), st in zip(jobs, streams):
+                blk.launch(p, st.cuda_stream)
+        torch.cuda.synchronize()
+        for blk, raw, x, p, out, alone in jobs:
+            assert all(torch.equal(o, a) for o, a in zip(out, alone))
