@@ -376,6 +376,32 @@ def test_block_random_long_buckets(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
         assert err <= OUT_TOL, (flags, err)
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "mxfp4"])
+@pytest.mark.parametrize("T,zipf_s", [(1000, 8.0), (257, 10.0)])
+def test_block_extreme_routing_skew(pkg, wl, oracle, dev, T, zipf_s, fmt):
+    """A router bias that sends nearly every token to the same four experts: buckets as long as the batch
+    next to empty and one-row buckets, through every kernel family; oracle on 200 tokens."""
+    shape = wl.MoeShape("skew", T=T, H=512, I=256, E=32, K=4, fmt=fmt, zipf_s=zipf_s, seed=3)
+    table = oracle.normal_table()
+    blk, raw = wl.make_device_layer(shape, table, dev)
+    x = wl.make_device_input(shape, table, dev)
+    hw = hostgen.host_layer(oracle, wl, shape)
+    sub = np.sort(np.random.default_rng(0).choice(T, min(T, 200), replace=False))
+    ref_y, ref_i, ref_v, _ = hostgen.oracle_block(oracle, shape, hw, hostgen.host_input(oracle, wl, shape)[sub])
+    for flags in (0, pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH,
+                  pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT, pkg.MOE_FLAG_FORCE_TILED):
+        y, ti, tv = blk.forward(x, flags=flags)
+        torch.cuda.synchronize()
+        counts = np.bincount(ti.cpu().numpy().ravel(), minlength=shape.E)
+        assert counts.max() >= 0.9 * T and (counts == 0).sum() >= 16   # the skew is what the test is about
+        assert np.array_equal(ti.cpu().numpy()[sub], ref_i), flags
+        np.testing.assert_allclose(tv.cpu().numpy()[sub], ref_v, rtol=2e-6)
+        err = hostgen.rel_err(y.cpu().numpy()[sub], ref_y)
+        assert err <= OUT_TOL, (flags, err)
+    say("  skew T=%d %s: longest bucket %d rows, %d empty experts, rel err %.2e" %
+        (T, fmt, counts.max(), (counts == 0).sum(), err))
+
+
 def test_block_residual_and_rmsnorm_glue(pkg, wl, oracle, dev):
     shape = wl.MoeShape("glue", T=40, H=256, I=128, E=8, K=4, fmt="bf16", seed=3)
     table = oracle.normal_table()
