@@ -1316,11 +1316,14 @@ MOE_DEVICE void prefill_body_mxfp4(const ExpertGemmArgs& a, uint8_t* lds, int e,
         wait_vmcnt<0>();  // next stage's activations (direct-to-LDS) and weights have landed
         __syncthreads();
     };
-    issue_b(0);
+    // weights, scales and biases first: their addresses need the tile's expert only, while the activation
+    // loads wait for the token ids of the tile's rows (one memory round trip more)
     load_scales(sw_cur, 0);
     load_a(0, 0);
     uint2 bias_raw[R];  // fetched with the first stage: its latency stays off the block's tail
     load_bias<R>(a, e, unit, 0, bias_raw);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_b(0);
     wait_vmcnt<0>();
     __syncthreads();
     for (int qd = 0; qd < n_quads; ++qd) {
