@@ -23,6 +23,7 @@ MOE_FLAG_FORCE_STREAM = 2
 MOE_FLAG_FORCE_TILED = 4
 MOE_FLAG_FORCE_DIRECT = 8
 MOE_FLAG_FORCE_BUCKET_LAUNCH = 16
+MOE_FLAG_FUSED_GEMM_LAUNCH = 32
 
 _c = ctypes
 _vp, _i, _ll, _f, _u, _sz = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float, _c.c_uint, _c.c_size_t

@@ -47,6 +47,15 @@ inline bool use_direct_bucketing(int T, int K, int E, bool prefill, unsigned fla
     return A <= 48LL * E;
 }
 
+// Both expert GEMMs in one launch: on request, when the bucketing is done inside the expert kernels and
+// the experts fit the kernel's per-XCD tables.  Measured at the 20b decode shape it ties with the two
+// launches for bf16 weights (what it saves in launch boundaries it pays for emptying and refilling its
+// pipeline where a down item has to wait for its expert's gate/up items) and is slower for MXFP4,
+// whose stages are a quarter as long; so it is not the default.
+inline bool use_fused_experts(int E, bool direct, unsigned flags) {
+    return direct && (flags & MOE_FLAG_FUSED_GEMM_LAUNCH) && E <= expert_fused_max_experts();
+}
+
 // Carves the caller's workspace for moe_block_forward; with base == nullptr only sizes it.
 struct BlockWorkspace {
     double* router_partial;
@@ -59,6 +68,7 @@ struct BlockWorkspace {
     int* tile_row0;
     int* tile_rows;
     int* n_tiles;          // [1]
+    int* fused_ctr;        // counters of the one-launch expert kernel (experts_fused.hip)
     uint16_t* h_by_slot;   // [A, I] bf16 SwiGLU outputs
     float* y_by_slot;      // [A, H] fp32 down-projection rows
     int max_tiles;
@@ -85,6 +95,7 @@ struct BlockWorkspace {
         tile_row0 = static_cast<int*>(take((size_t)2 * max_tiles * 4));
         tile_rows = static_cast<int*>(take((size_t)2 * max_tiles * 4));
         n_tiles = static_cast<int*>(take(4));
+        fused_ctr = static_cast<int*>(take((size_t)expert_fused_ctr_words(E) * 4));
         h_by_slot = static_cast<uint16_t*>(take(A * I * 2));
         y_by_slot = static_cast<float*>(take(A * H * 4));
         bytes = off;
@@ -500,6 +511,27 @@ struct ExpertPlan {
             }
         }
     }
+    // One launch for both GEMMs: row blocks per expert (n1 gate/up, n2 down, at most the kernel's consumer
+    // waves in row units each).  A block's time is its number of items (an item's ticks take about the same
+    // time whatever its rows), so: as few rounds of items over an XCD's compute units as possible, and among
+    // those the split that leaves the fewest compute units without an item in the last round.
+    void pick_fused(int* n1, int* n2, int* drain_slack) const {
+        const int cons = expert_fused_consumers();
+        const int U1 = 2 * p->intermediate_dim / 32, U2 = p->hidden_dim / 32;
+        const int per_xcd = std::max(1, ceil_div(p->n_experts, 8)), cus = std::max(1, n_cus / 8);
+        long long best = -1;
+        for (int a = ceil_div(U1, cons); a <= ceil_div(U1, cons) + 4; ++a)
+            for (int b = ceil_div(U2, cons); b <= ceil_div(U2, cons) + 4; ++b) {
+                const int items = per_xcd * (a + b), rounds = ceil_div(items, cus);
+                const long long cost = (long long)rounds * 1000000 + (long long)(rounds * cus - items) * 100 + a + b;
+                if (best < 0 || cost < best) {
+                    best = cost;
+                    *n1 = a;
+                    *n2 = b;
+                }
+            }
+        *drain_slack = 2 * cus;  // two rounds of items
+    }
     void set_weights(ExpertGemmArgs& a, const void* w, const void* scales, int rows, int Kdim) const {
         a.w = w;
         a.w_scales = static_cast<const uint8_t*>(scales);
@@ -631,16 +663,30 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     if ((rc = mark())) return rc;
 
     // 3. gate/up GEMM + SwiGLU  (src/forward.cpp:474-479; src/run.cpp:657-689)
+    // 4. down GEMM  (src/forward.cpp:481-487; src/run.cpp:691-700)
     const ExpertPlan plan(p, ws, prefill, direct, tile_tokens, max_tiles);
     const ExpertGemmArgs a1 = plan.gate_up(ws.t_bf16, ws.h_by_slot);
-    rc = launch_expert_stream(a1, 0, stream);
-    if (rc) return rc;
-    if ((rc = mark())) return rc;
-
-    // 4. down GEMM  (src/forward.cpp:481-487; src/run.cpp:691-700)
     const ExpertGemmArgs a2 = plan.down(ws.h_by_slot, ws.y_by_slot);
-    rc = launch_expert_stream(a2, 1, stream);
-    if (rc) return rc;
+    if (use_fused_experts(E, direct, p->flags)) {
+        // one launch for both (its stage time is reported as the gate/up stage, the down stage is empty)
+        ExpertFusedArgs f{};
+        f.gu = a1;
+        f.dn = a2;
+        f.ctr = ws.fused_ctr;
+        f.spin_limit = 1 << 20;
+        plan.pick_fused(&f.n1, &f.n2, &f.drain_slack);
+        rc = launch_fill_zero(reinterpret_cast<uint32_t*>(ws.fused_ctr), expert_fused_ctr_words(E), stream);
+        if (rc) return rc;
+        rc = launch_expert_fused(f, plan.n_cus, stream);
+        if (rc) return rc;
+        if ((rc = mark())) return rc;
+    } else {
+        rc = launch_expert_stream(a1, 0, stream);
+        if (rc) return rc;
+        if ((rc = mark())) return rc;
+        rc = launch_expert_stream(a2, 1, stream);
+        if (rc) return rc;
+    }
     if ((rc = mark())) return rc;
 
     // 5. weighted combine in ascending expert id (+ residual)  (src/run.cpp:702-712)
@@ -658,6 +704,7 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
     }
     return mark();
 }
+
 
 int moe_block_forward(const moe_block_params* p, moe_stream_t stream) { return block_forward_impl(p, stream, nullptr); }
 
@@ -702,8 +749,13 @@ int moe_block_describe(const moe_block_params* p, char* text, size_t text_bytes)
         }
     };
     char g1[96], g2[96];
-    gemm_name(2 * I, 0, g1, sizeof(g1));
-    gemm_name(H, 1, g2, sizeof(g2));
+    if (use_fused_experts(E, direct, p->flags)) {
+        snprintf(g1, sizeof(g1), "expert_fused_kernel<%d>", fmt);
+        snprintf(g2, sizeof(g2), "expert_fused_kernel<%d>", fmt);
+    } else {
+        gemm_name(2 * I, 0, g1, sizeof(g1));
+        gemm_name(H, 1, g2, sizeof(g2));
+    }
     const int n = snprintf(text, text_bytes, "router=%s; bucketing=%s; gate_up=%s; down=%s; combine=%s; compute_units=%d",
                            router, direct ? "in the expert kernels" : "bucket_kernel", g1, g2,
                            p->next_norm_out ? "combine_norm_kernel" : "combine_kernel", plan.n_cus);

@@ -104,6 +104,22 @@ struct ExpertGemmArgs {
 int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream);
 int expert_direct_max_assignments();
 
+// ---- experts_fused.hip: both expert GEMMs of a block in one launch (bucketing inside the kernel) --
+struct ExpertFusedArgs {
+    ExpertGemmArgs gu, dn;  // the gate/up and the down GEMM as launch_expert_stream would get them
+    int* ctr;               // expert_fused_ctr_words() ints, all zero at launch: [0..7] item queue heads per XCD,
+                            // [8] set when a bounded wait ran out, [16 + e] finished gate/up items of expert e
+    int n1, n2;             // row blocks per expert of the gate/up and of the down GEMM
+    int drain_slack;        // a gate/up item is counted as finished at once when fewer queue positions than this lie
+                            // between its expert's last gate/up item and first down item
+    int spin_limit;         // quads a block keeps looking for a finished-items count before it gives up
+};
+inline int expert_fused_ctr_words(int n_experts) { return 16 + n_experts; }
+int expert_fused_max_assignments();
+int expert_fused_max_experts();
+int expert_fused_consumers();
+int launch_expert_fused(const ExpertFusedArgs& f, int n_blocks, hipStream_t stream);
+
 // ---- combine.hip -------------------------------------------------------------------------------
 int launch_combine(const float* y_by_slot, const int* slot_of, const int* topk_i, const float* topk_v,
                    float* e_agg, float* residual_x, int T, int K, int H, hipStream_t stream);
@@ -116,6 +132,7 @@ int launch_rmsnorm(float* o, const float* x, const uint16_t* weight, int batch, 
 
 // ---- mxfp4.hip ---------------------------------------------------------------------------------
 void mxfp4_tiled_bytes(int rows, int K, size_t* block_bytes, size_t* scale_bytes);
+int launch_fill_zero(uint32_t* words, size_t n, hipStream_t stream);
 int launch_dequant_mxfp4(const uint8_t* blocks, const uint8_t* scales, long long n_blocks, uint16_t* out,
                          hipStream_t stream);
 int launch_mxfp4_repack(const uint8_t* blocks, const uint8_t* scales, int E, int rows, int K,

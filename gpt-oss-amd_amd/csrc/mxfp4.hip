@@ -101,6 +101,12 @@ __global__ void fill_zero_kernel(uint32_t* __restrict__ p, size_t n) {
     if (i < n) p[i] = 0u;
 }
 
+int launch_fill_zero(uint32_t* words, size_t n, hipStream_t stream) {
+    if (n == 0) return MOE_OK;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)ceil_div(n, (size_t)256)), dim3(256), 0, stream, words, n);
+    return launch_status();
+}
+
 int launch_mxfp4_repack(const uint8_t* blocks, const uint8_t* scales, int E, int rows, int K,
                         uint8_t* tiled_blocks, uint8_t* tiled_scales, bool inverse, hipStream_t stream) {
     const int G = K / 32;

@@ -324,7 +324,10 @@ enum {
     MOE_FLAG_FORCE_DIRECT = 8u,        /* weight-streaming kernels: bucket inside the expert kernels whenever
                                           the batch allows it (n_tokens * experts_per_token <= 4096,
                                           n_tokens <= 2048), however long the buckets */
-    MOE_FLAG_FORCE_BUCKET_LAUNCH = 16u /* always run the bucketing kernel and its token-block map */
+    MOE_FLAG_FORCE_BUCKET_LAUNCH = 16u, /* always run the bucketing kernel and its token-block map */
+    MOE_FLAG_FUSED_GEMM_LAUNCH = 32u   /* decode-sized batches (those that bucket inside the expert kernels),
+                                          n_experts <= 256: one launch for both expert GEMMs instead of one
+                                          each; ignored for other batches */
 };
 
 MOE_API size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int intermediate_dim, int n_experts,

@@ -68,3 +68,9 @@ def rel_err(y, ref):
     """max|y - ref| / max|ref| : the output tolerance metric (outputs cross zero, so an element-wise
     relative error has no meaning)."""
     return float(np.abs(y.astype(np.float64) - ref.astype(np.float64)).max() / np.abs(ref).max())
+
+
+def rms_err(y, ref):
+    """||y - ref||_2 / ||ref||_2 : the RMS-relative error reported beside the tolerance metric."""
+    d = y.astype(np.float64) - ref.astype(np.float64)
+    return float(np.sqrt((d * d).sum() / (ref.astype(np.float64) ** 2).sum()))

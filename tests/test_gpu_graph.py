@@ -9,9 +9,12 @@ pytestmark = pytest.mark.gpu
 
 # T, H, I, E, K, fmt -> bucketing inside the expert kernels / bucketing launch + 64-token blocks /
 # 128-token blocks (both MXFP4 and the two bf16 kernels) / two-pass router
+FUSED = 32  # MOE_FLAG_FUSED_GEMM_LAUNCH: both expert GEMMs in one launch (counters cleared by a kernel)
 CASES = [
     (64, 256, 128, 8, 4, "mxfp4"),
     (64, 256, 128, 8, 4, "bf16"),
+    (64, 256, 128, 8, 4, "mxfp4", FUSED),
+    (96, 320, 192, 16, 4, "bf16", FUSED),
     (300, 192, 128, 8, 1, "mxfp4"),
     (260, 320, 192, 4, 1, "bf16"),      # 65 rows per expert: two blocks a compute unit
     (700, 320, 192, 8, 4, "bf16"),      # 350 rows per expert: one block a compute unit
@@ -22,8 +25,11 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("T,H,I,E,K,fmt", CASES)
-def test_graph_replays_equal_the_eager_call(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "-".join(str(v) for v in c))
+def test_graph_replays_equal_the_eager_call(pkg, wl, oracle, dev, case):
+    T, H, I, E, K, fmt = case[:6]
+    flags = case[6] if len(case) > 6 else 0
+    assert FUSED == pkg.MOE_FLAG_FUSED_GEMM_LAUNCH
     shape = wl.MoeShape("graph", T=T, H=H, I=I, E=E, K=K, fmt=fmt, seed=5 + T)
     table = oracle.normal_table()
     blk, raw = wl.make_device_layer(shape, table, dev)
@@ -33,7 +39,7 @@ def test_graph_replays_equal_the_eager_call(pkg, wl, oracle, dev, T, H, I, E, K,
     ti = torch.empty((T, K), dtype=torch.int32, device=dev)
     tv = torch.empty((T, K), dtype=torch.float32, device=dev)
     x_in = x.clone()
-    p = blk.params(x_in, e_agg, ti, tv)
+    p = blk.params(x_in, e_agg, ti, tv, flags=flags)
     stream = torch.cuda.current_stream().cuda_stream
     print("graph", shape, blk.describe(p), flush=True)
 

@@ -257,15 +257,22 @@ def test_block_small(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
     assert torch.equal(ti2, ti) and torch.equal(y2, y) and torch.equal(tv2, tv)
     # both kernel families on every shape, and the streaming family with either way of bucketing
     # (inside the expert kernels / by the bucketing launch), whichever the size rule picked above
+    by_family = {}
     for name, flag in (("64-token blocks, bucketing in the expert kernels",
                         pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT),
+                       ("both GEMMs in one launch",
+                        pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT | pkg.MOE_FLAG_FUSED_GEMM_LAUNCH),
                        ("64-token blocks, bucketing launch",
                         pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH),
                        ("128-token blocks", pkg.MOE_FLAG_FORCE_TILED)):
         yf, tif, _ = blk.forward(x, flags=flag)
         errf = hostgen.rel_err(yf.cpu().numpy(), ref_y)
-        say("  %s: rel err %.3e" % (name, errf))
+        say("  %s: rel err %.3e rms %.3e" % (name, errf, hostgen.rms_err(yf.cpu().numpy(), ref_y)))
         assert torch.equal(tif, ti) and errf <= OUT_TOL
+        by_family[name] = yf
+    # the one-launch kernel multiplies and adds in the order of the two-launch kernels: same bits
+    assert torch.equal(by_family["both GEMMs in one launch"],
+                       by_family["64-token blocks, bucketing in the expert kernels"])
 
 
 @pytest.mark.parametrize("T,H", [(40, 256), (130, 2880), (9, 4160)])
@@ -330,6 +337,7 @@ def test_block_random_shapes(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
     hw = hostgen.host_layer(oracle, wl, shape)
     ref_y, ref_i, ref_v, _ = hostgen.oracle_block(oracle, shape, hw, hostgen.host_input(oracle, wl, shape))
     for flags in (0, pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT,
+                  pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT | pkg.MOE_FLAG_FUSED_GEMM_LAUNCH,
                   pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH, pkg.MOE_FLAG_FORCE_TILED):
         y, ti, tv = blk.forward(x, flags=flags)
         torch.cuda.synchronize()
@@ -367,6 +375,7 @@ def test_block_random_long_buckets(pkg, wl, oracle, dev, T, H, I, E, K, fmt):
     families = [0, pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH, pkg.MOE_FLAG_FORCE_TILED]
     if T * K <= 4096:  # the longest assignment list a block scans itself
         families.append(pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT)
+        families.append(pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT | pkg.MOE_FLAG_FUSED_GEMM_LAUNCH)
     for flags in families:
         y, ti, tv = blk.forward(x, flags=flags)
         torch.cuda.synchronize()
@@ -389,7 +398,9 @@ def test_block_extreme_routing_skew(pkg, wl, oracle, dev, T, zipf_s, fmt):
     sub = np.sort(np.random.default_rng(0).choice(T, min(T, 200), replace=False))
     ref_y, ref_i, ref_v, _ = hostgen.oracle_block(oracle, shape, hw, hostgen.host_input(oracle, wl, shape)[sub])
     for flags in (0, pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH,
-                  pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT, pkg.MOE_FLAG_FORCE_TILED):
+                  pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT,
+                  pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT | pkg.MOE_FLAG_FUSED_GEMM_LAUNCH,
+                  pkg.MOE_FLAG_FORCE_TILED):
         y, ti, tv = blk.forward(x, flags=flags)
         torch.cuda.synchronize()
         counts = np.bincount(ti.cpu().numpy().ravel(), minlength=shape.E)
