@@ -84,13 +84,14 @@ inline int read_inputfile(const char* input_filename, int max_token_len, int max
 }
 
 // src/getp/eval.cpp:81-100.  One line per request: its generated tokens up to the first negative
-// entry, separated by single spaces.
+// entry, separated by single spaces.  A request's slot holds max_seq_len + 1 entries: the walk stops
+// there even without a terminator (the reference walks on into the next request's slot).
 inline int write_outputfile(const char* output_filename, Requests* reqs) {
     std::ofstream out(output_filename);
     if (!out.is_open()) return MOE_ERR_IO;
     for (int i = 0; i < reqs->num_reqs; i++) {
         const int* output_tokens = get_tok_gen_ptr(reqs, i);
-        for (int j = 0; output_tokens[j] >= 0; j++) {
+        for (int j = 0; j <= reqs->max_seq_len && output_tokens[j] >= 0; j++) {
             if (j > 0) out << ' ';
             out << output_tokens[j];
         }
@@ -160,6 +161,11 @@ struct DecodeOptions {
     int vocab = 64;       // that many consecutive values of an output row stand in for the logits
     int eos_token = -1;   // a sampled token equal to this ends its sequence (the reference: 199999, 200002)
     bool record_steps = false;
+    // If not NULL, every step is appended as: int32 {valid_batch_size, window}, int32 indices[valid],
+    // int32 tokens_in[valid], float rows_in[valid, hidden], float rows_out[valid, hidden],
+    // int32 tokens_out[valid] (the token each sequence takes next), so that a test can follow the loop
+    // step by step.  Costs two device-to-host copies per step.
+    FILE* trace = nullptr;
 };
 
 // Device and pinned host buffers of one worker (the reference's ThreadLocalBatchBuffers,
@@ -257,8 +263,10 @@ inline long long generate(moe_host::OssMoeTransformer* t_d, DecodeBuffers* buffe
             finished[b_idx] = 1;
             active_sequences--;
             if (output_tokens_batch[b_idx]) {
+                // a sequence that runs out of steps inside its prompt has generated nothing: the terminator
+                // goes to entry 0 (the reference writes none then, and its writer walks past the slot)
                 const int end_idx = pos[b_idx] - n_prompt + 1;
-                if (end_idx >= 0) output_tokens_batch[b_idx][end_idx] = -1;
+                output_tokens_batch[b_idx][end_idx >= 0 ? end_idx : 0] = -1;
             }
         }
         current_tokens[b_idx] = next_token;
@@ -285,6 +293,14 @@ inline long long generate(moe_host::OssMoeTransformer* t_d, DecodeBuffers* buffe
             return -(long long)hipGetLastError();
         if ((rc = moe_gather_rows(buffers->x_seq_d, buffers->indices_d, t_d->state.x, valid_batch_size, H, t_d->stream)))
             return -(long long)rc;
+        std::vector<float> trace_rows;
+        if (opt.trace) {
+            trace_rows.resize((size_t)2 * valid_batch_size * H);
+            if (hipMemcpyAsync(trace_rows.data(), t_d->state.x, sizeof(float) * (size_t)valid_batch_size * H,
+                               hipMemcpyDeviceToHost, stream) != hipSuccess ||
+                hipStreamSynchronize(stream) != hipSuccess)
+                return -(long long)hipGetLastError();
+        }
         float* out = moe_host::forward(t_d, buffers->tokens, buffers->positions, valid_batch_size, buffers->indices,
                                        t_d->config.batch_size);  // :588
         if (!out) return -(long long)t_d->last_error;
@@ -298,6 +314,16 @@ inline long long generate(moe_host::OssMoeTransformer* t_d, DecodeBuffers* buffe
                              sizeof(float) * opt.vocab, valid_batch_size, hipMemcpyDeviceToHost, stream) != hipSuccess)
             return -(long long)hipGetLastError();
         if (hipStreamSynchronize(stream) != hipSuccess) return -(long long)hipGetLastError();
+        if (opt.trace) {
+            if (hipMemcpy(trace_rows.data() + (size_t)valid_batch_size * H, out, sizeof(float) * (size_t)valid_batch_size * H,
+                          hipMemcpyDeviceToHost) != hipSuccess)
+                return -(long long)hipGetLastError();
+            const int head[2] = {valid_batch_size, window};
+            fwrite(head, sizeof(int), 2, opt.trace);
+            fwrite(buffers->indices, sizeof(int), valid_batch_size, opt.trace);
+            fwrite(buffers->tokens, sizeof(int), valid_batch_size, opt.trace);
+            fwrite(trace_rows.data(), sizeof(float), trace_rows.size(), opt.trace);
+        }
 
         for (int i = 0; i < valid_batch_size; i++) {  // :603-617
             const int b_idx = buffers->indices[i];
@@ -311,6 +337,11 @@ inline long long generate(moe_host::OssMoeTransformer* t_d, DecodeBuffers* buffe
                     if (logits[v] > logits[next_token]) next_token = v;
                 commit_generation(b_idx, next_token, true);
             }
+        }
+        if (opt.trace) {
+            std::vector<int> taken(valid_batch_size);
+            for (int i = 0; i < valid_batch_size; i++) taken[i] = current_tokens[buffers->indices[i]];
+            fwrite(taken.data(), sizeof(int), valid_batch_size, opt.trace);
         }
     }
     if (final_rows_h) {

@@ -7,7 +7,7 @@
 // Usage:
 //   moe_stack_main layers <ckpt> <bin_f32|bin_bf16|safetensors:K> <x.f32> <T> <out.f32> [flags]
 //   moe_stack_main getp   <ckpt> <bin_f32|bin_bf16|safetensors:K> <in.txt> <out.txt> <steps> <batch> <vocab> <eos>
-//                         [<final_states.f32> [<step_sizes.txt>]]
+//                         [<final_states.f32> [<step_sizes.txt> [<trace.bin>]]]   (trace: DecodeOptions::trace)
 //   moe_stack_main requests <in.txt> <out.txt> <max_seq_len> [truncate]     (file formats only, no device)
 //   moe_stack_main verify <generated.txt> <ground_truth.txt>
 // MXFP4 files stay MXFP4 on the device (tiled layout); dense files are uploaded as bf16.
@@ -177,10 +177,15 @@ static int run_getp(int argc, char** argv) {
     CHECK_RC(load_model(argv[2], argv[3], batch, &m));
     moe_getp::Requests reqs;
     CHECK_RC(moe_getp::read_inputfile(argv[4], /*max_token_len=*/8, steps, &reqs, 0));
+    if (argc > 12) {
+        opt.trace = std::fopen(argv[12], "wb");
+        if (!opt.trace) return 3;
+    }
     moe_getp::DecodeBuffers buffers;
     std::vector<int> step_sizes;
     std::vector<float> finals((size_t)reqs.num_reqs * m.tr.config.hidden_dim);
     const long long n_tokens = moe_getp::inference(&m.tr, &buffers, &reqs, steps, opt, &step_sizes, finals.data());
+    if (opt.trace) std::fclose(opt.trace);
     if (n_tokens < 0) CHECK_RC(-n_tokens);
     CHECK_RC(moe_getp::write_outputfile(argv[5], &reqs));
     std::printf("getp: %d requests, batch %d, %lld tokens generated, %zu steps\n", reqs.num_reqs, batch, n_tokens,

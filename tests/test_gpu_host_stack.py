@@ -2,8 +2,9 @@
 __graft_entry__.build()): a checkpoint file written here goes through moe_host::moe_upload_weights,
 moe_host::forward_layers / forward() (the reference's per-step entry, src/forward.cpp:202-204) and the
 decode loop of host/moe_getp.hpp (src/getp/run.cpp:467-659).  The residual stream after every layer is
-compared with the CPU oracle; the decode loop's tokens and final states must not depend on the batch
-size (compaction of the live batch, src/getp/run.cpp:573-588)."""
+compared with the CPU oracle; the decode loop is followed step by step by a Python restatement of
+src/getp/run.cpp:545-617 over the oracle's layer function, and its tokens and final states must not depend
+on the batch size (compaction of the live batch, src/getp/run.cpp:573-588)."""
 import os
 import subprocess
 
@@ -107,3 +108,166 @@ def test_cpp_decode_loop_is_batch_invariant(dev, tmp_path):
         assert text == text8
         assert np.array_equal(fin.view(np.uint32), fin8.view(np.uint32)), "state rows depend on the batch size"
         assert max(sizes) <= batch
+
+
+# ---- the decode loop against an oracle-side loop -----------------------------------------------------
+
+def initial_state_row(request, H):
+    """The stand-in for a prompt's embedding (host/moe_getp.hpp): FNV-1a of the bytes seeds a 32-bit xorshift."""
+    h = 2166136261
+    for c in request.encode():
+        h = ((h ^ c) * 16777619) & 0xFFFFFFFF
+    if h == 0:
+        h = 1
+    row = np.empty(H, dtype=np.float32)
+    for i in range(H):
+        h ^= (h << 13) & 0xFFFFFFFF
+        h ^= h >> 17
+        h ^= (h << 5) & 0xFFFFFFFF
+        row[i] = np.float32(h - (1 << 32) if h >= (1 << 31) else h) * np.float32(1.0 / 2147483648.0)
+    return row
+
+
+def oracle_generate(prompts, steps, vocab, eos, H, forward):
+    """generate() of the reference's batch runtime (src/getp/run.cpp:467-659) for one batch, restated:
+    prompt tokens are the request's bytes, sequence b owns state row b, a step runs `forward(step, indices,
+    rows_in)` on the rows of the sequences still running, and commit_generation (:545-571) gives each its
+    next prompt token or the first maximum of the moving logit window, and ends it at the end token or when
+    the steps run out.  Returns (outputs, step_sizes, per-step records, final rows)."""
+    B = len(prompts)
+    prompt_tokens = [list(p.encode()) or [0] for p in prompts]
+    rows = np.stack([initial_state_row(p, H) for p in prompts])
+    current = [pt[0] for pt in prompt_tokens]
+    pos = [0] * B
+    finished = [False] * B
+    out = [[] for _ in range(B)]
+    step_sizes, records = [], []
+    active = B
+
+    def commit(b, token, counted):
+        nonlocal active
+        if counted and pos[b] - len(prompt_tokens[b]) >= 0:
+            out[b].append(token)
+        if (token == eos or pos[b] + 1 >= steps) and not finished[b]:
+            finished[b] = True
+            active -= 1
+        current[b] = token
+
+    it = 0
+    while active > 0:
+        idx = [b for b in range(B) if not finished[b] and pos[b] + 1 < steps]      # :573-583
+        if not idx:
+            break
+        step_sizes.append(len(idx))
+        tokens_in = [current[b] for b in idx]
+        rows_in = rows[idx].copy()
+        rows_out = forward(len(records), idx, rows_in)
+        rows[idx] = rows_out
+        window = (it * vocab) % (H - vocab + 1)
+        it += 1
+        margins = []
+        for i, b in enumerate(idx):                                                   # :603-617
+            pos[b] += 1
+            if pos[b] < len(prompt_tokens[b]):
+                commit(b, prompt_tokens[b][pos[b]], False)
+                margins.append(np.inf)
+            else:
+                logits = rows_out[i, window:window + vocab]
+                top = int(np.argmax(logits))                                          # first maximum
+                rest = np.delete(logits, top)
+                margins.append(float(logits[top] - rest.max()) if len(rest) else np.inf)
+                commit(b, top, True)
+        records.append(dict(indices=idx, window=window, tokens_in=tokens_in, rows_in=rows_in, rows_out=rows_out,
+                            tokens_out=[current[b] for b in idx], margins=margins))
+    return out, step_sizes, records, rows
+
+
+def read_trace(path, H):
+    raw = np.fromfile(path, dtype=np.int32)
+    steps, o = [], 0
+    while o < len(raw):
+        n, window = int(raw[o]), int(raw[o + 1])
+        o += 2
+        idx = raw[o:o + n].tolist(); o += n
+        tok_in = raw[o:o + n].tolist(); o += n
+        rin = raw[o:o + n * H].view(np.float32).reshape(n, H); o += n * H
+        rout = raw[o:o + n * H].view(np.float32).reshape(n, H); o += n * H
+        tok_out = raw[o:o + n].tolist(); o += n
+        steps.append(dict(indices=idx, window=window, tokens_in=tok_in, rows_in=rin, rows_out=rout, tokens_out=tok_out))
+    return steps
+
+
+LONG_PROMPTS = PROMPTS + ["a prompt that is longer than the step budget allows!"]
+
+
+def test_cpp_decode_loop_vs_oracle_loop(oracle, dev, tmp_path):
+    """`moe_stack_main getp` with a step trace against the loop restated in Python over oracle.moe_layer:
+    (1) fed the GPU's own rows as forward results, the restated loop must reproduce the GPU program's live
+    batches, tokens, step sizes and output file exactly (the loop logic, no arithmetic involved);
+    (2) every step's rows: the oracle's layers on the GPU's input rows give the GPU's output rows within the
+    block tolerance, and wherever the oracle's logit window has a margin above twice that row's error the GPU
+    sampled the oracle's token;  (3) a prompt that does not fit the step budget generates nothing and leaves
+    an empty line."""
+    path, kind, tensors = write_model(tmp_path, "mxfp4")
+    H, L, K = CFG["hidden_size"], CFG["num_hidden_layers"], CFG["experts_per_token"]
+    prompts = LONG_PROMPTS
+    with open(tmp_path / "in.txt", "w") as f:
+        f.write("%d\n" % len(prompts))
+        f.writelines(p + "\n" for p in prompts)
+    steps, vocab, eos, batch = 28, 8, 3, len(prompts)
+    r = run("getp", path, kind, tmp_path / "in.txt", tmp_path / "out.txt", steps, batch, vocab, eos, tmp_path / "fin.f32",
+            tmp_path / "sz.txt", tmp_path / "trace.bin")
+    assert r.returncode == 0, r.stdout + r.stderr
+    trace = read_trace(tmp_path / "trace.bin", H)
+    gpu_sizes = [int(v) for v in open(tmp_path / "sz.txt").read().split()]
+    gpu_lines = open(tmp_path / "out.txt").read().split("\n")[:-1]
+    gpu_tokens = [[int(t) for t in l.split()] for l in gpu_lines]
+    gpu_final = np.fromfile(tmp_path / "fin.f32", dtype=np.float32).reshape(len(prompts), H)
+    assert len(gpu_lines) == len(prompts) and len(trace) == len(gpu_sizes)
+    # the request file reader cuts a line to its slot of 8 x (steps + 1) - 1 characters: none is that long here
+    assert gpu_tokens[-1] == [], "a prompt as long as the step budget generates nothing"
+
+    # (1) the loop logic, replaying the GPU's rows
+    def replay(step, idx, rows_in):
+        assert idx == trace[step]["indices"], ("live batch differs at step", step)
+        assert np.array_equal(rows_in, trace[step]["rows_in"]), ("state rows differ at step", step)
+        return trace[step]["rows_out"]
+
+    out, sizes, records, final = oracle_generate(prompts, steps, vocab, eos, H, replay)
+    assert sizes == gpu_sizes
+    assert out == gpu_tokens
+    assert np.array_equal(final, gpu_final)
+    for rec, tr in zip(records, trace):
+        assert rec["window"] == tr["window"] and rec["tokens_in"] == tr["tokens_in"] and rec["tokens_out"] == tr["tokens_out"]
+
+    # (2) the arithmetic of every step against the oracle's layers
+    weights = [layer_weights(tensors, l, True) for l in range(L)]
+
+    def oracle_forward(x):
+        for w in weights:
+            x = oracle.moe_layer(x, *w, K)[0]
+        return x
+
+    worst, decided, undecided = 0.0, 0, 0
+    for rec in records:
+        ref = oracle_forward(rec["rows_in"])
+        gpu = rec["rows_out"]
+        err = float(np.abs(gpu - ref).max() / np.abs(ref - rec["rows_in"]).max())
+        worst = max(worst, err)
+        assert err <= OUT_TOL, err
+        w = rec["window"]
+        for i, m in enumerate(rec["margins"]):
+            if not np.isfinite(m):
+                continue  # a prompt token was taken
+            logits = ref[i, w:w + vocab]
+            top = int(np.argmax(logits))
+            margin = float(logits[top] - np.delete(logits, top).max())
+            row_err = float(np.abs(gpu[i] - ref[i]).max())
+            if margin > 2 * row_err:
+                assert rec["tokens_out"][i] == top
+                decided += 1
+            else:
+                undecided += 1
+    print("  decode loop: %d steps, worst rel err of a step %.3e, %d sampled tokens pinned by the oracle, %d too close "
+          "to call" % (len(records), worst, decided, undecided), flush=True)
+    assert decided > 4 * max(1, undecided)
