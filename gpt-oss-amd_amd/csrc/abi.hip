@@ -204,27 +204,13 @@ int moe_bucket_by_expert(const int* topk_i, const float* topk_v, int B, int K, i
 int moe_gather_rows(const float* X, const int* idx, float* Y, int rows, int H, moe_stream_t stream) {
     if (!X || !idx || !Y) return MOE_ERR_NULL;
     if (rows <= 0 || H <= 0 || H % 4 != 0) return MOE_ERR_SHAPE;
-    if (rows > 65535) {
-        // grid.y limit: split into slabs
-        for (int r0 = 0; r0 < rows; r0 += 65535) {
-            int rc = launch_gather_rows(X, idx + r0, Y + (size_t)r0 * H, rows - r0 < 65535 ? rows - r0 : 65535, H,
-                                        as_stream(stream));
-            if (rc) return rc;
-        }
-        return MOE_OK;
-    }
-    return launch_gather_rows(X, idx, Y, rows, H, as_stream(stream));
+    return launch_gather_rows(X, idx, Y, rows, H, as_stream(stream));  // slabs of 65535 rows inside
 }
 
 int moe_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, moe_stream_t stream) {
     if (!X || !idx || !Y) return MOE_ERR_NULL;
     if (rows <= 0 || H <= 0 || H % 4 != 0) return MOE_ERR_SHAPE;
-    for (int r0 = 0; r0 < rows; r0 += 65535) {  // grid.y limit: slabs
-        int rc = launch_scatter_rows(Y + (size_t)r0 * H, idx + r0, X, rows - r0 < 65535 ? rows - r0 : 65535, H,
-                                     as_stream(stream));
-        if (rc) return rc;
-    }
-    return MOE_OK;
+    return launch_scatter_rows(Y, idx, X, rows, H, as_stream(stream));  // slabs of 65535 rows inside
 }
 
 int moe_count_tokens_per_expert(const int* topk_i, const float* topk_v, int B, int K, int* out_expert, int* out_token,
@@ -771,8 +757,12 @@ void moe_synth_normal_table(float* h_table) {
 int moe_block_down_gemm(const moe_block_params* caller, const moe_bf16_t* h_by_assignment, float* y_by_assignment,
                         moe_stream_t stream_) {
     if (!caller || !h_by_assignment || !y_by_assignment) return MOE_ERR_NULL;
-    if (caller->struct_bytes != sizeof(moe_block_params)) return MOE_ERR_FORMAT;
-    const moe_block_params* p = caller;
+    // as moe_block_forward: the struct as it was before next_norm_weight / next_norm_out is still accepted
+    constexpr size_t kOldBytes = offsetof(moe_block_params, next_norm_weight);
+    if (caller->struct_bytes != sizeof(moe_block_params) && caller->struct_bytes != kOldBytes) return MOE_ERR_FORMAT;
+    moe_block_params local{};
+    memcpy(&local, caller, caller->struct_bytes);
+    const moe_block_params* p = &local;
     const int T = p->n_tokens, H = p->hidden_dim, I = p->intermediate_dim, E = p->n_experts,
               K = p->experts_per_token;
     int rc = check_dims(T, H, I, E, K);

@@ -191,10 +191,17 @@ __global__ void gather_rows_kernel(const float4* __restrict__ X, const int* __re
     Y[(size_t)row * H4 + c] = X[(size_t)idx[row] * H4 + c];
 }
 
+// One grid row per table row: launched in slabs of kMaxGridRows rows (the grid's y limit).
+constexpr int kMaxGridRows = 65535;
+
 int launch_gather_rows(const float* X, const int* idx, float* Y, int rows, int H, hipStream_t stream) {
     const int H4 = H / 4;
-    hipLaunchKernelGGL(gather_rows_kernel, dim3(ceil_div(H4, 256), rows), dim3(256), 0, stream,
-                       reinterpret_cast<const float4*>(X), idx, reinterpret_cast<float4*>(Y), rows, H4);
+    for (int r0 = 0; r0 < rows; r0 += kMaxGridRows) {
+        const int n = rows - r0 < kMaxGridRows ? rows - r0 : kMaxGridRows;
+        hipLaunchKernelGGL(gather_rows_kernel, dim3(ceil_div(H4, 256), n), dim3(256), 0, stream,
+                           reinterpret_cast<const float4*>(X), idx + r0, reinterpret_cast<float4*>(Y) + (size_t)r0 * H4, n,
+                           H4);
+    }
     return launch_status();
 }
 
@@ -210,8 +217,12 @@ __global__ void scatter_rows_kernel(const float4* __restrict__ Y, const int* __r
 
 int launch_scatter_rows(const float* Y, const int* idx, float* X, int rows, int H, hipStream_t stream) {
     const int H4 = H / 4;
-    hipLaunchKernelGGL(scatter_rows_kernel, dim3(ceil_div(H4, 256), rows), dim3(256), 0, stream,
-                       reinterpret_cast<const float4*>(Y), idx, reinterpret_cast<float4*>(X), rows, H4);
+    for (int r0 = 0; r0 < rows; r0 += kMaxGridRows) {
+        const int n = rows - r0 < kMaxGridRows ? rows - r0 : kMaxGridRows;
+        hipLaunchKernelGGL(scatter_rows_kernel, dim3(ceil_div(H4, 256), n), dim3(256), 0, stream,
+                           reinterpret_cast<const float4*>(Y) + (size_t)r0 * H4, idx + r0, reinterpret_cast<float4*>(X), n,
+                           H4);
+    }
     return launch_status();
 }
 

@@ -1,9 +1,11 @@
 // The reference's per-step entry of the GPU path,
 //   float* forward(OssTransformerHybrid*, OssExpertParallelGroup*, int* tokens, const int* pos_per_token_h,
 //                  int batch_size, const int* batch_indices_h, int B_stride)      (src/forward.cpp:202-204),
-// for the part of the model this library covers: the MoE half of every layer on one GPU.  The
-// expert-parallel group is gone (one GPU, no peers); every other argument keeps its place and meaning,
-// so the decode loop of the getp runtime (src/getp/run.cpp:573-588) can call it unchanged.
+// for the part of the model this library covers: the MoE half of every layer on one GPU.  Both forms
+// exist: the reference's own seven arguments, where the expert-parallel group must describe this one GPU
+// (NULL, or ep_size 1: one GPU, no peers; anything else is MOE_ERR_FORMAT), so that the call in the decode
+// loop of the getp runtime (src/getp/run.cpp:588) compiles and runs unchanged; and the same without the
+// group.
 //
 // What it runs, for l = 0 .. n_layers-1 on the compact batch of `batch_size` rows of s->x:
 //   t = rmsnorm(x, rms_ffn_w[l]);  e_agg = moe(t);  x += e_agg          (src/forward.cpp:315-514)
@@ -38,50 +40,14 @@ inline int forward_layers(OssMoeTransformer* tr, int batch_size, int first, int 
     const OssMoeRunState& s = tr->state;
     if (batch_size <= 0 || batch_size > p.batch_size || first < 0 || last > p.n_layers || first > last)
         return MOE_ERR_SHAPE;
-    const long long H = p.hidden_dim, I = p.intermediate_dim, E = p.n_experts;
-    size_t b1 = 0, s1 = 0, b2 = 0, s2 = 0;
-    if (w.w_mlp1_blocks) {
-        moe_mxfp4_tiled_bytes(2 * p.intermediate_dim, p.hidden_dim, &b1, &s1);
-        moe_mxfp4_tiled_bytes(p.hidden_dim, p.intermediate_dim, &b2, &s2);
-    }
+    const long long H = p.hidden_dim;
     for (int l = first; l < last; ++l) {
         if (l == first && !norm_ready) {
             const int rc = moe_rmsnorm(s.t, s.x, w.rms_ffn_w + l * H, batch_size, p.hidden_dim, tr->stream);
             if (rc) return rc;
         }
-        moe_block_params bp{};
-        bp.struct_bytes = sizeof(bp);
-        bp.n_tokens = batch_size;
-        bp.hidden_dim = p.hidden_dim;
-        bp.intermediate_dim = p.intermediate_dim;
-        bp.n_experts = p.n_experts;
-        bp.experts_per_token = p.experts_per_token;
-        bp.swiglu_limit = p.swiglu_limit;
-        bp.alpha = 1.702f;  // literal in the reference: src/run.cpp:673, src/forward.cpp:467
-        bp.t = s.t;
-        bp.w_router = w.w_router + l * E * H;
-        bp.b_router = w.b_router + l * E;
-        bp.b_mlp1 = w.b_mlp1 + l * E * 2 * I;
-        bp.b_mlp2 = w.b_mlp2 + l * E * H;
-        if (w.w_mlp1_blocks) {
-            bp.weight_format = MOE_WEIGHTS_MXFP4_TILED;
-            bp.w_mlp1 = w.w_mlp1_blocks + (size_t)l * E * b1;
-            bp.w_mlp1_scales = w.w_mlp1_scales + (size_t)l * E * s1;
-            bp.w_mlp2 = w.w_mlp2_blocks + (size_t)l * E * b2;
-            bp.w_mlp2_scales = w.w_mlp2_scales + (size_t)l * E * s2;
-        } else {
-            bp.weight_format = MOE_WEIGHTS_BF16;
-            bp.w_mlp1 = w.w_mlp1 + l * E * 2 * I * H;
-            bp.w_mlp2 = w.w_mlp2 + l * E * H * I;
-        }
-        bp.e_agg = s.e_agg;
-        bp.topk_i = s.topk_i;
-        bp.topk_v = s.topk_v;
-        bp.router_score = s.router_score;
-        bp.residual_x = s.x;
-        bp.workspace = s.workspace;
-        bp.workspace_bytes = s.workspace_bytes;
-        bp.flags = tr->flags;
+        moe_block_params bp;
+        moe_fill_block_params(p, w, s, l, batch_size, tr->flags, &bp);
         if (l + 1 < last) {  // the next layer's FFN norm, written by this block's last kernel
             bp.next_norm_weight = w.rms_ffn_w + (l + 1) * H;
             bp.next_norm_out = s.t;
@@ -94,6 +60,15 @@ inline int forward_layers(OssMoeTransformer* tr, int batch_size, int first, int 
 
 // One layer, for a caller that runs its own attention half between the MoE halves.
 inline int forward_layer(OssMoeTransformer* tr, int l, int batch_size) { return forward_layers(tr, batch_size, l, l + 1); }
+
+// include/model.hpp:264-269: what forward() reads of the reference's expert-parallel context.  This
+// library runs every expert on the caller's GPU, so a group can only name that one GPU.
+struct OssExpertParallelGroup {
+    void** shards = nullptr;       // the reference's shard descriptors; never read here
+    int dp_rank = 0;
+    int ep_size = 1;               // number of shards: must be 1
+    int primary_shard_index = 0;
+};
 
 // src/forward.cpp:202-204 without the expert-parallel group.
 inline float* forward(OssMoeTransformer* transformer, int* tokens, const int* pos_per_token_h, int batch_size,
@@ -122,6 +97,17 @@ inline float* forward(OssMoeTransformer* transformer, int* tokens, const int* po
         return nullptr;
     }
     return transformer->state.x;
+}
+
+// src/forward.cpp:202-204, argument for argument.
+inline float* forward(OssMoeTransformer* transformer, OssExpertParallelGroup* ep_group, int* tokens,
+                      const int* pos_per_token_h, int batch_size, const int* batch_indices_h, int B_stride) {
+    if (!transformer) return nullptr;
+    if (ep_group && ep_group->ep_size != 1) {  // the reference exits on an invalid context (:209-212)
+        transformer->last_error = MOE_ERR_FORMAT;
+        return nullptr;
+    }
+    return forward(transformer, tokens, pos_per_token_h, batch_size, batch_indices_h, B_stride);
 }
 
 }  // namespace moe_host

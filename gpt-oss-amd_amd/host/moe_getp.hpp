@@ -166,6 +166,9 @@ struct DecodeOptions {
     // int32 tokens_out[valid] (the token each sequence takes next), so that a test can follow the loop
     // step by step.  Costs two device-to-host copies per step.
     FILE* trace = nullptr;
+    // the reference's thread-local expert-parallel group (src/getp/run.cpp:136), handed to forward() as there;
+    // NULL or a group of one shard
+    moe_host::OssExpertParallelGroup* ep_group = nullptr;
 };
 
 // Device and pinned host buffers of one worker (the reference's ThreadLocalBatchBuffers,
@@ -301,8 +304,8 @@ inline long long generate(moe_host::OssMoeTransformer* t_d, DecodeBuffers* buffe
                 hipStreamSynchronize(stream) != hipSuccess)
                 return -(long long)hipGetLastError();
         }
-        float* out = moe_host::forward(t_d, buffers->tokens, buffers->positions, valid_batch_size, buffers->indices,
-                                       t_d->config.batch_size);  // :588
+        float* out = moe_host::forward(t_d, opt.ep_group, buffers->tokens, buffers->positions, valid_batch_size,
+                                       buffers->indices, t_d->config.batch_size);  // :588
         if (!out) return -(long long)t_d->last_error;
         if ((rc = moe_scatter_rows(out, buffers->indices_d, buffers->x_seq_d, valid_batch_size, H, t_d->stream)))
             return -(long long)rc;

@@ -6,9 +6,12 @@
 // Differences a caller sees:
 //   * errors come back as return codes (0 = ok) instead of exit(1) inside CHECK_HIP
 //     (include/model.hpp:8-17);
-//   * gemm_router needs a scratch buffer (fp64 partial sums): pass one through
-//     moe_router_scratch(), sized by moe_router_scratch_bytes(); without one the call goes to
-//     moe_gemm_router_static (fixed 16 MiB array inside the library, N * M limited);
+//   * gemm_router needs a scratch buffer (fp64 partial sums): register one per host thread through
+//     moe_router_scratch(), sized by moe_router_scratch_bytes(); without one the call returns
+//     MOE_ERR_WORKSPACE.  A caller that cannot provide one (graph capture, no allocation allowed) may opt
+//     into the fixed array inside the library with moe_router_scratch().use_static_array = true: that
+//     array is one per GPU, so only ONE stream of ONE host thread per GPU may then run gemm_router at a
+//     time (two calls that overlap on a GPU mix their partial sums and return wrong logits, silently);
 //   * bucketing is one call (bucket_by_expert) instead of memset + three kernels
 //     (src/forward.cpp:333-349), and there is one work queue instead of a heavy and a light one;
 //   * __hip_bfloat16 pointers are passed as moe_bf16_t* (same size and bit layout).
@@ -20,6 +23,7 @@ namespace moe_dropin {
 struct RouterScratch {
     void* ptr = nullptr;
     size_t bytes = 0;
+    bool use_static_array = false;  // no buffer: fall back to moe_gemm_router_static (one call per GPU at a time!)
 };
 // one scratch registration per host thread, matching the reference's thread-per-GPU model
 // (src/getp/run.cpp:680-692); the library itself keeps no state
@@ -32,9 +36,10 @@ inline RouterScratch& moe_router_scratch() {
 inline int gemm_router(float* xout, const float* x_batch, const moe_bf16_t* w, const moe_bf16_t* bias, int N, int K,
                        int M, moe_stream_t stream = nullptr) {
     RouterScratch& s = moe_router_scratch();
-    // no registered buffer: the variant whose scratch is a fixed array inside the library
-    if (!s.ptr) return moe_gemm_router_static(xout, x_batch, w, bias, N, K, M, stream);
-    return moe_gemm_router(xout, x_batch, w, bias, N, K, M, s.ptr, s.bytes, stream);
+    if (s.ptr) return moe_gemm_router(xout, x_batch, w, bias, N, K, M, s.ptr, s.bytes, stream);
+    // no registered buffer: an error, unless the caller asked for the library's fixed array (see above)
+    if (!s.use_static_array) return MOE_ERR_WORKSPACE;
+    return moe_gemm_router_static(xout, x_batch, w, bias, N, K, M, stream);
 }
 
 // src/hip/topk.hip:59-60

@@ -104,15 +104,11 @@ inline size_t moe_workspace_bytes(const OssMoeConfig& p) {
     return moe_block_workspace_bytes(p.batch_size, p.hidden_dim, p.intermediate_dim, p.n_experts, p.experts_per_token);
 }
 
-// One layer's FFN half, the counterpart of src/forward.cpp:315-514 on a single GPU:
-//   t = rmsnorm(x, rms_ffn_w[l]);  e_agg = moe(t);  x += e_agg
-// Everything is queued on `stream`; nothing waits for the device (the reference blocks on a D2H copy
-// of the expert offsets once per layer, src/forward.cpp:340-345, 381).
-inline int moe_forward_layer(const OssMoeConfig& p, const OssMoeWeights& w, const OssMoeRunState& s, int l,
-                             int batch_size, moe_stream_t stream, unsigned flags = 0) {
+// The argument block of moe_block_forward for layer l: one layer's slices of the stacked tensors
+// (src/forward.cpp:317-514 addresses them the same way: base + l * per-layer size).
+inline void moe_fill_block_params(const OssMoeConfig& p, const OssMoeWeights& w, const OssMoeRunState& s, int l,
+                                  int batch_size, unsigned flags, moe_block_params* out) {
     const long long H = p.hidden_dim, I = p.intermediate_dim, E = p.n_experts;
-    int rc = moe_rmsnorm(s.t, s.x, w.rms_ffn_w + l * H, batch_size, p.hidden_dim, stream);
-    if (rc) return rc;
     moe_block_params bp{};
     bp.struct_bytes = sizeof(bp);
     bp.n_tokens = batch_size;
@@ -149,6 +145,19 @@ inline int moe_forward_layer(const OssMoeConfig& p, const OssMoeWeights& w, cons
     bp.workspace = s.workspace;
     bp.workspace_bytes = s.workspace_bytes;
     bp.flags = flags;
+    *out = bp;
+}
+
+// One layer's FFN half, the counterpart of src/forward.cpp:315-514 on a single GPU:
+//   t = rmsnorm(x, rms_ffn_w[l]);  e_agg = moe(t);  x += e_agg
+// Everything is queued on `stream`; nothing waits for the device (the reference blocks on a D2H copy
+// of the expert offsets once per layer, src/forward.cpp:340-345, 381).
+inline int moe_forward_layer(const OssMoeConfig& p, const OssMoeWeights& w, const OssMoeRunState& s, int l,
+                             int batch_size, moe_stream_t stream, unsigned flags = 0) {
+    const int rc = moe_rmsnorm(s.t, s.x, w.rms_ffn_w + (long long)l * p.hidden_dim, batch_size, p.hidden_dim, stream);
+    if (rc) return rc;
+    moe_block_params bp;
+    moe_fill_block_params(p, w, s, l, batch_size, flags, &bp);
     return moe_block_forward(&bp, stream);
 }
 

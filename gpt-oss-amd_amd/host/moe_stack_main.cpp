@@ -8,6 +8,9 @@
 //   moe_stack_main layers <ckpt> <bin_f32|bin_bf16|safetensors:K> <x.f32> <T> <out.f32> [flags]
 //   moe_stack_main getp   <ckpt> <bin_f32|bin_bf16|safetensors:K> <in.txt> <out.txt> <steps> <batch> <vocab> <eos>
 //                         [<final_states.f32> [<step_sizes.txt> [<trace.bin>]]]   (trace: DecodeOptions::trace)
+//   moe_stack_main dropin <ckpt> <bin_f32|bin_bf16> <x.f32> <T> <out.f32> <scratch: own|static|none>
+//           every layer's MoE half issued call by call, in the reference's order (src/forward.cpp:315-514),
+//           through the reference-named wrappers of moe_kernels.hpp; residual stream written out per layer
 //   moe_stack_main requests <in.txt> <out.txt> <max_seq_len> [truncate]     (file formats only, no device)
 //   moe_stack_main verify <generated.txt> <ground_truth.txt>
 // MXFP4 files stay MXFP4 on the device (tiled layout); dense files are uploaded as bf16.
@@ -20,6 +23,7 @@
 #include <vector>
 
 #include "moe_getp.hpp"
+#include "moe_kernels.hpp"
 
 #define CHECK_RC(expr)                                                                      \
     do {                                                                                    \
@@ -164,6 +168,118 @@ static int run_layers(int argc, char** argv) {
         return 4;
     }
     std::printf("forward() equals the layer-by-layer result bit for bit\n");
+    // the reference's seven-argument form: a group of one shard runs, a group of two is refused
+    moe_host::OssExpertParallelGroup one, two;
+    two.ep_size = 2;
+    if (moe_host::forward(&m.tr, &two, tokens.data(), pos.data(), T, idx.data(), T) != nullptr ||
+        m.tr.last_error != MOE_ERR_FORMAT) {
+        std::fprintf(stderr, "forward() accepted an expert-parallel group of two shards\n");
+        return 4;
+    }
+    std::vector<float> x1;
+    CHECK_RC(read_floats(argv[4], &x1, n));
+    CHECK_RC(hipMemcpy(m.tr.state.x, x1.data(), n * sizeof(float), hipMemcpyHostToDevice));
+    y = moe_host::forward(&m.tr, &one, tokens.data(), pos.data(), T, idx.data(), T);
+    if (!y) CHECK_RC(m.tr.last_error);
+    CHECK_RC(hipDeviceSynchronize());
+    CHECK_RC(hipMemcpy(x1.data(), y, n * sizeof(float), hipMemcpyDeviceToHost));
+    if (std::memcmp(x1.data(), x.data(), n * sizeof(float)) != 0) {
+        std::fprintf(stderr, "the seven-argument forward() differs\n");
+        return 4;
+    }
+    std::printf("forward() with the reference's seven arguments: same bits; a group of two shards is refused\n");
+    return 0;
+}
+
+// The MoE half of every layer the way the reference's layer loop issues it (src/forward.cpp:315-514):
+// rmsnorm, gemm_router, topk, softmax, the three bucketing kernels, gather_rows, the work queue, the two
+// expert GEMMs, vecadd_and_zero — each through its reference-named wrapper.  `scratch`: "own" registers a
+// router scratch buffer for this thread, "static" opts into the library's fixed array, "none" does neither
+// (gemm_router must then refuse with MOE_ERR_WORKSPACE).
+static int run_dropin(int argc, char** argv) {
+    if (argc < 8) return 2;
+    const int T = std::atoi(argv[5]);
+    const std::string scratch = argv[7];
+    Model m;
+    CHECK_RC(load_model(argv[2], argv[3], T, &m));
+    const moe_host::OssMoeConfig& c = m.tr.config;
+    const moe_host::OssMoeWeights& w = m.tr.weights;
+    const moe_host::OssMoeRunState& s = m.tr.state;
+    if (w.w_mlp1_blocks) {
+        std::fprintf(stderr, "dropin: the reference-named wrappers take bf16 experts\n");
+        return 2;
+    }
+    const long long H = c.hidden_dim, I = c.intermediate_dim, E = c.n_experts, K = c.experts_per_token;
+    const size_t A = (size_t)T * K, n = (size_t)T * H;
+    float *router_score, *x_by_expert, *gate_by_expert, *assign_w, *weights_flat;
+    int *assign_expert, *assign_token, *expert_counts, *expert_offsets, *tokens_flat, *work_queue, *work_count;
+    void* router_scratch = nullptr;
+    CHECK_RC(dev_alloc(&router_score, (size_t)T * E));
+    CHECK_RC(dev_alloc(&x_by_expert, A * H));
+    CHECK_RC(dev_alloc(&gate_by_expert, A * I));
+    CHECK_RC(dev_alloc(&assign_w, A));
+    CHECK_RC(dev_alloc(&weights_flat, A));
+    CHECK_RC(dev_alloc(&assign_expert, A));
+    CHECK_RC(dev_alloc(&assign_token, A));
+    CHECK_RC(dev_alloc(&expert_counts, (size_t)E));
+    CHECK_RC(dev_alloc(&expert_offsets, (size_t)E + 1));
+    CHECK_RC(dev_alloc(&tokens_flat, A));
+    CHECK_RC(dev_alloc(&work_queue, (size_t)3 * E));
+    CHECK_RC(dev_alloc(&work_count, 1));
+    m.owned.insert(m.owned.end(), {router_score, x_by_expert, gate_by_expert, assign_w, weights_flat, assign_expert,
+                                   assign_token, expert_counts, expert_offsets, tokens_flat, work_queue, work_count});
+    if (scratch == "own") {
+        const size_t bytes = moe_router_scratch_bytes(T, (int)E);
+        CHECK_RC(hipMalloc(&router_scratch, bytes));
+        m.owned.push_back(router_scratch);
+        moe_dropin::moe_router_scratch().ptr = router_scratch;
+        moe_dropin::moe_router_scratch().bytes = bytes;
+    } else if (scratch == "static") {
+        moe_dropin::moe_router_scratch().use_static_array = true;
+    }
+    std::vector<float> x;
+    CHECK_RC(read_floats(argv[4], &x, n));
+    CHECK_RC(hipMemcpy(s.x, x.data(), n * sizeof(float), hipMemcpyHostToDevice));
+    CHECK_RC(hipMemset(s.e_agg, 0, n * sizeof(float)));          // zero on entry, re-zeroed by vecadd_and_zero
+    CHECK_RC(hipMemset(expert_counts, 0, sizeof(int) * E));      // zero on entry, reset by the scan
+    FILE* out = std::fopen(argv[6], "wb");
+    if (!out) return 3;
+    using namespace moe_dropin;
+    for (int l = 0; l < c.n_layers; ++l) {
+        CHECK_RC(rmsnorm(s.t, s.x, w.rms_ffn_w + l * H, T, (int)H));
+        const int rc = gemm_router(router_score, s.t, w.w_router + l * E * H, w.b_router + l * E, T, (int)H, (int)E);
+        if (scratch == "none") {
+            std::printf("gemm_router without a scratch buffer -> %d (%s)\n", rc, moe_error_string(rc));
+            std::fclose(out);
+            return rc == MOE_ERR_WORKSPACE ? 0 : 4;
+        }
+        CHECK_RC(rc);
+        CHECK_RC(topk(s.topk_v, s.topk_i, router_score, T, (int)E, (int)K));
+        CHECK_RC(softmax(s.topk_v, T, (int)K));
+        CHECK_RC(count_tokens_per_expert(s.topk_i, s.topk_v, T, (int)K, assign_expert, assign_token, assign_w,
+                                         expert_counts, (int)E));
+        CHECK_RC(exclusive_scan_expert_offsets(expert_counts, expert_offsets, (int)E));
+        CHECK_RC(compact_by_expert_kernel(assign_expert, assign_token, assign_w, (int)A, expert_offsets, expert_counts,
+                                          tokens_flat, weights_flat, (int)E));
+        // the compaction counted its writes in expert_counts; the reference zeroes them again for the next layer
+        CHECK_RC(hipMemsetAsync(expert_counts, 0, sizeof(int) * E, nullptr));
+        CHECK_RC(gather_rows(s.t, tokens_flat, x_by_expert, (int)A, (int)H));
+        CHECK_RC(build_work_queue(expert_offsets, (int)E, work_queue, work_count));
+        int n_work = 0;
+        CHECK_RC(hipMemcpy(&n_work, work_count, sizeof(int), hipMemcpyDeviceToHost));  // the reference's one D2H copy
+        CHECK_RC(moe_dropin::moe_mlp1_swiglu(work_queue, 0, n_work, x_by_expert, gate_by_expert, w.w_mlp1 + l * E * 2 * I * H,
+                                             w.b_mlp1 + l * E * 2 * I, (int)H, (int)I, 2 * I * H, 2 * I, 1.702f,
+                                             c.swiglu_limit, T, 0));
+        CHECK_RC(moe_dropin::moe_mlp2_scatter(work_queue, 0, n_work, gate_by_expert, tokens_flat, weights_flat, s.e_agg,
+                                              w.w_mlp2 + l * E * H * I, w.b_mlp2 + l * E * H, (int)I, (int)H, H * I, H, T,
+                                              0));
+        CHECK_RC(vecadd_and_zero(s.x, s.e_agg, 1.0f, T, (int)H));
+        CHECK_RC(hipDeviceSynchronize());
+        CHECK_RC(hipMemcpy(x.data(), s.x, n * sizeof(float), hipMemcpyDeviceToHost));
+        std::fwrite(x.data(), sizeof(float), n, out);
+    }
+    std::fclose(out);
+    std::printf("dropin: %d layers through the reference-named wrappers, router scratch: %s\n", c.n_layers, scratch.c_str());
     return 0;
 }
 
@@ -173,6 +289,8 @@ static int run_getp(int argc, char** argv) {
     moe_getp::DecodeOptions opt;
     opt.vocab = std::atoi(argv[8]);
     opt.eos_token = std::atoi(argv[9]);
+    moe_host::OssExpertParallelGroup group;  // one GPU: a group of one shard
+    opt.ep_group = &group;
     Model m;
     CHECK_RC(load_model(argv[2], argv[3], batch, &m));
     moe_getp::Requests reqs;
@@ -246,7 +364,8 @@ int main(int argc, char** argv) {
     if (argc >= 2 && std::string(argv[1]) == "requests") return run_requests(argc, argv);
     if (argc >= 2 && std::string(argv[1]) == "verify") return run_verify(argc, argv);
     if (argc >= 2 && std::string(argv[1]) == "layers") return run_layers(argc, argv);
+    if (argc >= 2 && std::string(argv[1]) == "dropin") return run_dropin(argc, argv);
     if (argc >= 2 && std::string(argv[1]) == "getp") return run_getp(argc, argv);
-    std::fprintf(stderr, "usage: %s layers|getp|requests|verify ... (see the head of moe_stack_main.cpp)\n", argv[0]);
+    std::fprintf(stderr, "usage: %s layers|dropin|getp|requests|verify ... (see the head of moe_stack_main.cpp)\n", argv[0]);
     return 2;
 }

@@ -9,6 +9,8 @@ scale addressing, in every kernel family.
 Screening bound: the two-pass router may only drop an expert whose approximate score is more than
 twice its error bound below the K-th best.  The bound is checked against exact scores on inputs made
 to stress it."""
+import zlib
+
 import numpy as np
 import pytest
 import torch
@@ -40,8 +42,10 @@ def routing(T, E, K, seed):
 # T, H, I, E, K : I is the contraction length of the down GEMM (320 = ragged last MX stage; 2880 real)
 # the last two: buckets of 100 / 200 rows (bf16: the 128-token-block kernel with one block a compute unit), whose
 # three-stage ring leaves two stages (2880 = 22.5 stages of 128) / one stage (448 = 3.5) after its whole turns
+# the last: 80 000 assignment rows, more than one grid dimension holds (the row moves into and out of slot order
+# run in slabs of 65535 rows)
 ONE_HOT = [(70, 128, 320, 8, 4), (33, 192, 2880, 4, 2), (300, 64, 320, 4, 4), (129, 2880, 2880, 8, 4),
-           (400, 2880, 2880, 8, 2), (200, 64, 448, 2, 2)]
+           (400, 2880, 2880, 8, 2), (200, 64, 448, 2, 2), (20000, 64, 64, 16, 4)]
 
 
 @pytest.mark.parametrize("fmt", ["mxfp4", "bf16"])
@@ -63,6 +67,8 @@ def test_one_hot_rows_through_the_block_down_gemm(pkg, wl, oracle, dev, T, H, I,
              "64-token blocks, bucketing in the expert kernels": pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_DIRECT,
              "64-token blocks, bucketing launch": pkg.MOE_FLAG_FORCE_STREAM | pkg.MOE_FLAG_FORCE_BUCKET_LAUNCH,
              "128-token blocks": pkg.MOE_FLAG_FORCE_TILED}
+    if A > 4096:  # past the longest assignment list a block scans itself: the flag is ignored, same path as the next
+        del flags["64-token blocks, bucketing in the expert kernels"]
     for name, f in flags.items():
         y = blk.down_gemm(ti_d, h, flags=f)
         torch.cuda.synchronize()
@@ -121,7 +127,8 @@ ADVERSARIAL = ["same sign", "wide range", "extreme rows", "near ties", "random"]
 def test_two_pass_router_bound_holds_with_margin(pkg, oracle, dev, T, H, E, K, case):
     """|approximate - exact| <= 0.5 * bound for every (token, expert): the screening pass may use the
     whole bound, so half of it is a safety factor of two."""
-    rng = np.random.default_rng(hash((T, E, case)) % (1 << 31))
+    # a seed that is the same in every process (str hashes are salted per process)
+    rng = np.random.default_rng(zlib.crc32(repr((T, E, case)).encode()))
     x = rng.standard_normal((T, H)).astype(np.float32)
     w = rng.standard_normal((E, H)) * 0.02
     b = rng.standard_normal(E) * 0.02

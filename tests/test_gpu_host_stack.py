@@ -61,6 +61,7 @@ def test_cpp_forward_layer_by_layer_vs_oracle(oracle, dev, tmp_path, fmt):
     r = run("layers", path, kind, tmp_path / "x.f32", T, tmp_path / "out.f32")
     assert r.returncode == 0, r.stdout + r.stderr
     assert "forward() equals the layer-by-layer result bit for bit" in r.stdout
+    assert "forward() with the reference's seven arguments: same bits; a group of two shards is refused" in r.stdout
     dump = np.fromfile(tmp_path / "out.f32", dtype=np.float32).reshape(L, T, H)
     x_in = x0
     for l in range(L):
@@ -70,6 +71,45 @@ def test_cpp_forward_layer_by_layer_vs_oracle(oracle, dev, tmp_path, fmt):
         print("  %s layer %d: rel err of the MoE contribution %.3e" % (fmt, l, err), flush=True)
         assert err <= OUT_TOL, (l, err)
         x_in = dump[l]
+
+
+@pytest.mark.parametrize("scratch", ["own", "static"])
+def test_cpp_dropin_wrappers_in_the_reference_call_order(oracle, dev, tmp_path, scratch):
+    """Every layer's MoE half issued call by call through the reference-named wrappers of host/moe_kernels.hpp
+    (gemm_router, topk, softmax, the three bucketing kernels, gather_rows, the work queue, moe_mlp1_swiglu,
+    moe_mlp2_scatter, vecadd_and_zero: src/forward.cpp:315-514), with a registered router scratch buffer and with
+    the library's fixed array; compared with the oracle layer by layer and with the one-call block."""
+    path, kind, tensors = write_model(tmp_path, "bin_bf16")
+    T, H, L, K = 45, CFG["hidden_size"], CFG["num_hidden_layers"], CFG["experts_per_token"]
+    x0 = (np.random.default_rng(2).standard_normal((T, H)) * 1.5).astype(np.float32)
+    x0.tofile(tmp_path / "x.f32")
+    r = run("dropin", path, kind, tmp_path / "x.f32", T, tmp_path / "dropin.f32", scratch)
+    assert r.returncode == 0, r.stdout + r.stderr
+    r2 = run("layers", path, kind, tmp_path / "x.f32", T, tmp_path / "layers.f32")
+    assert r2.returncode == 0, r2.stdout + r2.stderr
+    dump = np.fromfile(tmp_path / "dropin.f32", dtype=np.float32).reshape(L, T, H)
+    block = np.fromfile(tmp_path / "layers.f32", dtype=np.float32).reshape(L, T, H)
+    x_in = x0
+    for l in range(L):
+        ref_x, _, _ = oracle.moe_layer(x_in, *layer_weights(tensors, l, False), K)  # fed this path's own input
+        d_ref, d_gpu = ref_x - x_in, dump[l] - x_in
+        err = float(np.abs(d_gpu - d_ref).max() / np.abs(d_ref).max())
+        print("  dropin (%s scratch) layer %d: rel err of the MoE contribution %.3e" % (scratch, l, err), flush=True)
+        assert err <= OUT_TOL, (l, err)
+        x_in = dump[l]
+    # against the one-call block on the same input: the fp32 intermediate and the atomic combine order differ
+    d_blk, d_seq = block[0] - x0, dump[0] - x0
+    assert float(np.abs(d_seq - d_blk).max() / np.abs(d_blk).max()) <= 5e-3
+
+
+def test_cpp_dropin_router_refuses_without_a_scratch_buffer(dev, tmp_path):
+    """No registered buffer and no opt-in to the library's fixed array: gemm_router returns MOE_ERR_WORKSPACE."""
+    path, kind, _ = write_model(tmp_path, "bin_bf16")
+    T, H = 9, CFG["hidden_size"]
+    np.zeros((T, H), np.float32).tofile(tmp_path / "x.f32")
+    r = run("dropin", path, kind, tmp_path / "x.f32", T, tmp_path / "o.f32", "none")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "gemm_router without a scratch buffer -> -4" in r.stdout
 
 
 PROMPTS = ["abc", "hello", "xy", "prompt!", "q", "seven77", "ab", "longer one"]
