@@ -132,6 +132,94 @@ def test_safetensors_mxfp4(ck, tmp_path, fancy):
         assert np.array_equal(f.get_tensor("block.1.mlp.mlp2_weight.blocks"), tensors["block.1.mlp.mlp2_weight.blocks"])
 
 
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+REF_CFG = dict(ckptgen.TINY, hidden_size=128, intermediate_size=64, num_experts=8, num_hidden_layers=2)
+
+
+def ref_expected():
+    """What tests/golden/make_ref_bin.py fed the reference's exporter: the same generator, config and seed."""
+    tensors = ckptgen.make_tensors(REF_CFG, seed=11, mxfp4=True)
+    dense = {}
+    for n, a in tensors.items():
+        if n.endswith(".scales"):
+            continue
+        if n.endswith(".blocks"):
+            base = n[:-len(".blocks")]
+            dense[base] = ckptgen.mxfp4_dequant(a, tensors[base + ".scales"])
+        else:
+            dense[n] = a
+    return tensors, dense
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_reference_written_bin(ck, oracle, bf16):
+    """tests/golden/ref_tiny_{f32,bf16}.bin were written by the reference's own export_model_bin.py (its
+    dequantize_fp4, key order and header) from tests/golden/ref_tiny.safetensors.  The reader must find the
+    reference's config in the header and every MoE tensor at the offset the exporter put it, and the expert values
+    the exporter dequantised must be the ones the oracle's and the test generator's MXFP4 decoders give."""
+    import json
+    cfg = json.load(open(os.path.join(GOLDEN, "ref_tiny_config.json")))
+    assert cfg == REF_CFG
+    tensors, dense = ref_expected()
+    path = os.path.join(GOLDEN, "ref_tiny_bf16.bin" if bf16 else "ref_tiny_f32.bin")
+    raw = np.fromfile(path, dtype=np.uint8)
+    width = 2 if bf16 else 4
+    with ck.Checkpoint.open_bin(path, ck.DTYPE_BF16 if bf16 else ck.DTYPE_F32) as c:
+        got = c.config
+        for key, field in zip(ckptgen.CONFIG_KEYS, [f[0] for f in ck.CkptConfig._fields_]):
+            assert getattr(got, field) == cfg[key], key
+        assert not c.is_mxfp4 and len(c.tensors()) == 7 * 2
+        # the exporter's order, restated: header, then tensors grouped by kind with the layers in order inside
+        # each kind, so that the offsets of the MoE tensors depend on every tensor before them
+        offset = 4 * len(ckptgen.CONFIG_KEYS)
+        offsets = {}
+        for n in ckptgen.bin_order(list(dense)):
+            offsets[n] = offset
+            offset += dense[n].size * width
+        assert offset == raw.size
+        for l in range(2):
+            for which, name in enumerate(MOE_NAMES):
+                full = "block.%d.%s" % (l, name)
+                want = np.ascontiguousarray(dense[full], dtype=np.float32).ravel()
+                data, dtype = c.layer_tensor(l, which)
+                if bf16:
+                    assert dtype == ck.DTYPE_BF16 and np.array_equal(data, ckptgen.f32_to_bf16_bits(want)), full
+                else:
+                    assert dtype == ck.DTYPE_F32 and np.array_equal(data.view(np.uint32), want.view(np.uint32)), full
+                at = offsets[full]
+                assert np.array_equal(raw[at:at + want.size * width], np.ascontiguousarray(data).view(np.uint8)), full
+    # the oracle's decoder against the values the reference's dequantize_fp4 wrote (fp32 file: nothing rounded)
+    f32 = np.fromfile(os.path.join(GOLDEN, "ref_tiny_f32.bin"), dtype=np.uint8)
+    offset = 4 * len(ckptgen.CONFIG_KEYS)
+    for n in ckptgen.bin_order(list(dense)):
+        size = dense[n].size * 4
+        if n.endswith("mlp1_weight") or n.endswith("mlp2_weight"):
+            ref_vals = f32[offset:offset + size].view(np.float32)
+            bits = oracle.dequant_mxfp4(tensors[n + ".blocks"], tensors[n + ".scales"])
+            assert np.array_equal(ckptgen.f32_to_bf16_bits(ref_vals), bits.ravel()), n
+            assert np.array_equal(ckptgen.bf16_bits_to_f32(bits.ravel()), ref_vals), n
+        offset += size
+
+
+def test_reference_read_safetensors(ck):
+    """The safetensors file the reference's exporter read (tests/golden/ref_tiny.safetensors) through this reader:
+    same expert blocks and scales, dense tensors as BF16."""
+    tensors, _ = ref_expected()
+    with ck.Checkpoint.open_safetensors(os.path.join(GOLDEN, "ref_tiny.safetensors")) as c:
+        assert c.is_mxfp4
+        g = c.config
+        assert (g.hidden_dim, g.intermediate_dim, g.n_experts, g.n_layers) == (128, 64, 8, 2)
+        for l in range(2):
+            p = "block.%d.mlp." % l
+            for which, name in ((ck.T_W_MLP1, "mlp1_weight.blocks"), (ck.T_W_MLP1_SCALES, "mlp1_weight.scales"),
+                                (ck.T_W_MLP2, "mlp2_weight.blocks"), (ck.T_W_MLP2_SCALES, "mlp2_weight.scales")):
+                data, dtype = c.layer_tensor(l, which)
+                assert dtype == ck.DTYPE_U8 and np.array_equal(data, tensors[p + name].ravel())
+            for which, name in ((ck.T_RMS_FFN, "norm.scale"), (ck.T_B_MLP1, "mlp1_bias"), (ck.T_B_MLP2, "mlp2_bias")):
+                data, dtype = c.layer_tensor(l, which)
+                assert dtype == ck.DTYPE_BF16 and np.array_equal(data, ckptgen.f32_to_bf16_bits(tensors[p + name]).ravel())
+
+
 def test_safetensors_config_check_and_errors(ck, tmp_path):
     cfg = ckptgen.TINY
     tensors = ckptgen.make_tensors(cfg, seed=6, mxfp4=True)

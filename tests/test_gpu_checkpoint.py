@@ -1,6 +1,8 @@
 """GPU tests of the checkpoint reader: a file in either on-disk format, uploaded through
 moe_ckpt_upload_layer, must give the block the same weights bit for bit, and the block's output
 must match the CPU oracle run on the weights the test wrote."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -121,3 +123,45 @@ def test_upload_rejects_bad_arguments(pkg, ck, dev, tmp_path):
         d.struct_bytes = 8
         st = torch.empty(c.staging_bytes(), dtype=torch.uint8, device=dev)
         assert pkg.lib.moe_ckpt_upload_layer(c._h, 0, ctypes.byref(d), st.data_ptr(), st.numel(), None) == -5
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_reference_written_files_to_block(pkg, ck, oracle, dev):
+    """The files under tests/golden/ that the reference's export_model_bin.py read (ref_tiny.safetensors) and wrote
+    (ref_tiny_f32.bin, ref_tiny_bf16.bin, through its own dequantize_fp4): uploaded through the three routes
+    (.bin fp32, .bin bf16, safetensors dequantised on the device) every MoE tensor must come out as the same BF16
+    bits, and the three blocks must give the same output as the oracle on those weights."""
+    assert CFG == dict(ckptgen.TINY, hidden_size=128, intermediate_size=64, num_experts=8, num_hidden_layers=2)
+    tensors = ckptgen.make_tensors(CFG, seed=11, mxfp4=True)
+    want = ck.CkptConfig()
+    want.experts_per_token, want.swiglu_limit = CFG["experts_per_token"], CFG["swiglu_limit"]
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((41, 128)).astype(np.float32)
+    keys = ("w_router", "b_router", "w_mlp1", "b_mlp1", "w_mlp2", "b_mlp2", "rms_ffn_w")
+    with ck.Checkpoint.open_bin(os.path.join(GOLDEN, "ref_tiny_f32.bin"), ck.DTYPE_F32) as c32, \
+            ck.Checkpoint.open_bin(os.path.join(GOLDEN, "ref_tiny_bf16.bin"), ck.DTYPE_BF16) as c16, \
+            ck.Checkpoint.open_safetensors(os.path.join(GOLDEN, "ref_tiny.safetensors"), want) as cst:
+        for layer in (0, 1):
+            print("reference-written files, layer", layer, flush=True)
+            p = "block.%d.mlp." % layer
+            t32 = c32.upload_layer(layer, device=dev)
+            t16 = c16.upload_layer(layer, device=dev)
+            tst = cst.upload_layer(layer, device=dev, tiled=False)
+            for key in keys:
+                a, b, s = bits_of(t32[key]).ravel(), bits_of(t16[key]).ravel(), bits_of(tst[key]).ravel()
+                assert np.array_equal(a, b), key
+                assert np.array_equal(a, s), key  # device dequantiser == the reference's dequantize_fp4
+            assert np.array_equal(bits_of(t32["w_mlp1"]).ravel(),
+                                  oracle.dequant_mxfp4(tensors[p + "mlp1_weight.blocks"],
+                                                       tensors[p + "mlp1_weight.scales"]).ravel())
+            (ref_y, ref_i, ref_v, _), _ = oracle_layer(oracle, tensors, layer, x, CFG["experts_per_token"], True)
+            for name, c, kw in (("bin f32", c32, {}), ("bin bf16", c16, {}), ("safetensors tiled", cst, {"tiled": True})):
+                blk = c.moe_block(layer, max_tokens=64, device=dev, **kw)
+                y, ti, tv = blk.forward(torch.from_numpy(x).to(dev))
+                torch.cuda.synchronize()
+                assert np.array_equal(ti.cpu().numpy(), ref_i), name
+                err = hostgen.rel_err(y.cpu().numpy(), ref_y)
+                print("  %s: max-rel %.3g rms-rel %.3g" % (name, err, hostgen.rms_err(y.cpu().numpy(), ref_y)), flush=True)
+                assert err <= OUT_TOL, name
