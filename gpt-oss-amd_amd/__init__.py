@@ -114,6 +114,7 @@ SIGNATURES = {
     "moe_synth_normal_bf16": (_i, [_vp, _ll, _vp, _f, _u, _u, _vp]),
     "moe_synth_bytes": (_i, [_vp, _ll, _u, _u, _vp]),
     "moe_synth_range_bytes": (_i, [_vp, _ll, _u, _u, _u, _u, _vp]),
+    "moe_synth_checksum": (_i, [_vp, _ll, _vp, _vp]),
 }
 
 
@@ -483,6 +484,20 @@ def synth_normal_bf16(dst, table_d, scale, seed, tensor_id, stream=None):
 
 def synth_bytes(dst, seed, tensor_id, stream=None):
     _check("moe_synth_bytes", _lib.moe_synth_bytes(_ptr(dst), dst.numel(), seed, tensor_id, _stream(stream)))
+
+
+SYNTH_CHECKSUM_WORDS = 2049
+
+
+def synth_checksum(src, out=None, stream=None):
+    """Launches the checksum of `src` (any dtype, byte size a multiple of 16); returns the int64 device tensor whose
+    element 0 is the sum of the buffer's 32-bit words modulo 2^64 once the stream has run."""
+    import torch
+    if out is None:
+        out = torch.empty(SYNTH_CHECKSUM_WORDS, dtype=torch.int64, device=src.device)
+    _check("moe_synth_checksum", _lib.moe_synth_checksum(_ptr(src), src.numel() * src.element_size(), _ptr(out),
+                                                         _stream(stream)))
+    return out
 
 
 def synth_range_bytes(dst, seed, tensor_id, lo, span, stream=None):

@@ -857,4 +857,11 @@ int moe_synth_range_bytes(uint8_t* dst, long long n, unsigned seed, unsigned ten
     return launch_synth(3, dst, n, nullptr, 0.f, seed, tensor_id, lo, span, as_stream(stream));
 }
 
+int moe_synth_checksum(const void* src, long long n_bytes, unsigned long long* out_d, moe_stream_t stream) {
+    if (!src || !out_d) return MOE_ERR_NULL;
+    if (n_bytes <= 0 || (n_bytes & 15)) return MOE_ERR_SHAPE;
+    if (((uintptr_t)src & 15u) || ((uintptr_t)out_d & 7u)) return MOE_ERR_ALIGN;
+    return launch_synth_checksum(src, n_bytes, out_d, MOE_SYNTH_CHECKSUM_WORDS - 1, as_stream(stream));
+}
+
 }  // extern "C"

@@ -395,45 +395,52 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     if constexpr (FMT == FMT_BF16) {
-        // The contraction range is walked in pairs of MFMA steps (64 elements = one 128-byte
-        // line of a weight row): in a pair, lane group g takes elements 16g .. 16g+7 in the first
-        // step and 16g+8 .. 16g+15 in the second, so a lane's two 16-byte loads are adjacent and
-        // the four lane groups cover the whole line.  Ring of four pairs, loads issued three
-        // pairs (one and a half stages) ahead of their use; nothing touches a loaded value
-        // before the pair that consumes it.
+        // The contraction range is walked in pairs of MFMA steps (64 elements = one 128-byte line of a
+        // weight row).  A pair of a row tile is fetched by two instructions that each take WHOLE lines:
+        // instruction i holds tile rows 8i .. 8i+7, its lane (g, q) the 16-byte chunk 2g + (q >> 3) of tile
+        // row 8i + (q & 7).  Every line is then requested by one instruction only, which is what lets the
+        // loads be non-temporal (a line shared by two instructions is fetched twice under that hint) and
+        // takes the stream from the plain-load rate to the streaming rate of the memory system.  The MFMA
+        // operand of step h wants lane (g, q) to hold chunk 2g + h of tile row q: lanes 8..15 of every
+        // 16-lane row of instruction 0 and lanes 0..7 of instruction 1 trade places (row_ror:8 under a bank
+        // mask, in the stage that consumes the pair).  Ring of four pairs, loads issued three pairs (one
+        // and a half stages) ahead of their use; nothing touches a loaded value before that pair.
         constexpr int DP = 4;
         const int n_pairs = K / 64;
         const uint8_t* a_ptr[R];
         const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row = group * 64 + tile_row_in_group(r0 + r, q);
-            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 16 * g);
+            const int row = group * 64 + tile_row_in_group(r0 + r, q & 7);
+            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 8 * (2 * g + (q >> 3)));
         }
+        const size_t second_half = (size_t)32 * K * 2;  // tile row q + 8 is weight row + 32 (tile_row_in_group)
         u32x4 ar[DP][2][R];
         auto load_a = [&](int slot, int pair) {
             const size_t off = (size_t)(pair < n_pairs ? pair : 0) * 128;  // a padding pair re-reads pair 0 (unused)
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int r = 0; r < R; ++r)
-                    ar[slot][h][r] = *reinterpret_cast<const u32x4*>(a_ptr[r] + off + 16 * h);
+                    ar[slot][i][r] =
+                        __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a_ptr[r] + off + second_half * i));
         };
 #pragma unroll
         for (int i = 0; i < DP - 1; ++i) load_a(i, i);
         if constexpr (PRE) __syncthreads();
         __syncthreads();
-        // one stage = two pairs; `ss` (stage parity) fixes the ring slots at compile time
-        auto stage = [&](auto ss_tag, int st) {
+        // one stage = two pairs; `ss` (stage parity) fixes the ring slots at compile time.  HALF: the ragged
+        // last stage of a K that is an odd number of pairs runs its first pair only.
+        auto stage = [&](auto ss_tag, auto half_tag, int st) {
             constexpr int ss = decltype(ss_tag)::value;
+            constexpr bool HALF = decltype(half_tag)::value;
 #pragma unroll
-            for (int pp = 0; pp < 2; ++pp) {
+            for (int pp = 0; pp < (HALF ? 1 : 2); ++pp) {
                 constexpr int kSlots = DP;
                 const int u = 2 * ss + pp;  // ring slot of this pair
                 const int pair = 2 * st + pp;
                 load_a((u + kSlots - 1) % kSlots, pair + kSlots - 1);
                 __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three pairs ahead of their use
-                const bool live = pair < n_pairs;   // wave-uniform; false only in the second half of a ragged stage
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     u32x4 b[NT];
@@ -441,7 +448,13 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
                     for (int t = 0; t < NT; ++t) b[t] = b_frag(st, 2 * pp + h, t);
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
-                        const u32x4 av = live ? ar[u][h][r] : u32x4{0u, 0u, 0u, 0u};
+                        u32x4 av;
+#pragma unroll
+                        for (int d = 0; d < 4; ++d)
+                            av[d] = h == 0 ? (uint32_t)__builtin_amdgcn_update_dpp((int)ar[u][0][r][d], (int)ar[u][1][r][d],
+                                                                                   0x128, 0xF, 0xC, false)
+                                           : (uint32_t)__builtin_amdgcn_update_dpp((int)ar[u][1][r][d], (int)ar[u][0][r][d],
+                                                                                   0x128, 0xF, 0x3, false);
 #pragma unroll
                         for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
                     }
@@ -449,12 +462,18 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
             }
             __syncthreads();
         };
-        const int n_even = n_stages & ~1;
+        const int full_stages = n_pairs >> 1;
+        const int n_even = full_stages & ~1;
         for (int s0 = 0; s0 < n_even; s0 += 2) {
-            stage(std::integral_constant<int, 0>{}, s0);
-            stage(std::integral_constant<int, 1>{}, s0 + 1);
+            stage(std::integral_constant<int, 0>{}, std::false_type{}, s0);
+            stage(std::integral_constant<int, 1>{}, std::false_type{}, s0 + 1);
         }
-        if (n_stages & 1) stage(std::integral_constant<int, 0>{}, n_even);
+        if (full_stages & 1) {
+            stage(std::integral_constant<int, 0>{}, std::false_type{}, n_even);
+            if (n_pairs & 1) stage(std::integral_constant<int, 1>{}, std::true_type{}, n_even + 1);
+        } else if (n_pairs & 1) {
+            stage(std::integral_constant<int, 0>{}, std::true_type{}, n_even);
+        }
     } else {
         // Weights: a ring of four stages (one 128-bit load per row tile and stage, issued three
         // stages ahead of its use); scales: one word per row tile covers four stages and is

@@ -143,5 +143,8 @@ int launch_mxfp4_tiled_to_bf16(const uint8_t* tiled_blocks, const uint8_t* tiled
 // ---- synth.hip ---------------------------------------------------------------------------------
 int launch_synth(int kind, void* dst, long long n, const float* table, float scale, unsigned seed,
                  unsigned tensor_id, unsigned lo, unsigned span, hipStream_t stream);
+// out[0] = sum of the n_bytes / 16 * 4 32-bit words at src modulo 2^64; out[1 .. max_partials] is scratch.
+int launch_synth_checksum(const void* src, long long n_bytes, unsigned long long* out, int max_partials,
+                          hipStream_t stream);
 
 }  // namespace moe

@@ -11,11 +11,14 @@
 //   moe_stack_main dropin <ckpt> <bin_f32|bin_bf16> <x.f32> <T> <out.f32> <scratch: own|static|none>
 //           every layer's MoE half issued call by call, in the reference's order (src/forward.cpp:315-514),
 //           through the reference-named wrappers of moe_kernels.hpp; residual stream written out per layer
+//   moe_stack_main synth  <T> <H> <I> <E> <K> <layers> <steps> <warmup> [flags]
+//           a synthetic MXFP4 stack generated on the device, forward() timed over <steps> calls (one JSON line)
 //   moe_stack_main requests <in.txt> <out.txt> <max_seq_len> [truncate]     (file formats only, no device)
 //   moe_stack_main verify <generated.txt> <ground_truth.txt>
 // MXFP4 files stay MXFP4 on the device (tiled layout); dense files are uploaded as bf16.
 #include <hip/hip_runtime_api.h>
 
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -34,6 +37,10 @@
         }                                                                                   \
     } while (0)
 
+static double now_ms() {
+    return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
 template <typename T>
 static int dev_alloc(T** p, size_t count) {
     return (int)hipMalloc((void**)p, sizeof(T) * (count ? count : 1));
@@ -47,25 +54,11 @@ struct Model {
     }
 };
 
-// kind: bin_f32 | bin_bf16 | safetensors:<experts per token> (a safetensors file does not record it; the
-// reference's exporter takes it from config.json, tools/model_export/gpt-oss-20b/export_model_bin.py:302-304)
-static int load_model(const char* path, const std::string& kind, int batch_size, Model* m) {
-    moe_ckpt* ck = nullptr;
+// Stacked device tensors of every layer for m->tr.config (bf16 experts, or tiled MXFP4 ones), owned by `m`.
+static int alloc_weights(bool tiled, Model* m) {
+    const moe_host::OssMoeConfig& c = m->tr.config;
     int rc;
-    if (kind.rfind("safetensors", 0) == 0) {
-        moe_ckpt_config want{};  // shapes come from the file
-        want.experts_per_token = kind.size() > 12 ? std::atoi(kind.c_str() + 12) : 4;
-        want.swiglu_limit = 7.0f;
-        rc = moe_ckpt_open_safetensors(path, &want, &ck);
-    } else {
-        rc = moe_ckpt_open_bin(path, kind == "bin_bf16" ? MOE_DTYPE_BF16 : MOE_DTYPE_F32, &ck);
-    }
-    if (rc) return rc;
-    moe_host::OssMoeConfig& c = m->tr.config;
-    rc = moe_host::moe_config_from_checkpoint(ck, batch_size, &c);
-    if (rc) return rc;
     const size_t L = c.n_layers, E = c.n_experts, H = c.hidden_dim, I = c.intermediate_dim;
-    const bool tiled = moe_ckpt_is_mxfp4(ck) != 0;
     moe_host::OssMoeWeights& w = m->tr.weights;
     w = moe_host::OssMoeWeights{};
     moe_bf16_t *rms, *wr, *br, *b1, *b2, *w1 = nullptr, *w2 = nullptr;
@@ -97,17 +90,15 @@ static int load_model(const char* path, const std::string& kind, int batch_size,
     w.w_mlp1_scales = s1;
     w.w_mlp2_blocks = q2;
     w.w_mlp2_scales = s2;
-    const size_t staging_bytes = moe_ckpt_staging_bytes(ck);
-    uint8_t* staging;
-    if ((rc = dev_alloc(&staging, staging_bytes))) return rc;
-    rc = moe_host::moe_upload_weights(ck, c, w, staging, staging_bytes, nullptr);
-    if (!rc) rc = (int)hipDeviceSynchronize();
-    (void)hipFree(staging);
-    moe_ckpt_close(ck);
-    if (rc) return rc;
+    return MOE_OK;
+}
 
+// The run-state buffers for config.batch_size rows, owned by `m`.
+static int alloc_state(Model* m) {
+    const moe_host::OssMoeConfig& c = m->tr.config;
     moe_host::OssMoeRunState& s = m->tr.state;
-    const size_t B = batch_size;
+    const size_t B = c.batch_size, H = c.hidden_dim;
+    int rc;
     s.workspace_bytes = moe_host::moe_workspace_bytes(c);
     uint8_t* ws;
     if ((rc = dev_alloc(&s.x, B * H)) || (rc = dev_alloc(&s.t, B * H)) || (rc = dev_alloc(&s.e_agg, B * H)) ||
@@ -118,6 +109,38 @@ static int load_model(const char* path, const std::string& kind, int batch_size,
     s.router_score = nullptr;
     m->owned.insert(m->owned.end(), {s.x, s.t, s.e_agg, s.topk_v, s.topk_i, ws});
     return MOE_OK;
+}
+
+// kind: bin_f32 | bin_bf16 | safetensors:<experts per token> (a safetensors file does not record it; the
+// reference's exporter takes it from config.json, tools/model_export/gpt-oss-20b/export_model_bin.py:302-304)
+static int load_model(const char* path, const std::string& kind, int batch_size, Model* m) {
+    moe_ckpt* ck = nullptr;
+    int rc;
+    if (kind.rfind("safetensors", 0) == 0) {
+        moe_ckpt_config want{};  // shapes come from the file
+        want.experts_per_token = kind.size() > 12 ? std::atoi(kind.c_str() + 12) : 4;
+        want.swiglu_limit = 7.0f;
+        rc = moe_ckpt_open_safetensors(path, &want, &ck);
+    } else {
+        rc = moe_ckpt_open_bin(path, kind == "bin_bf16" ? MOE_DTYPE_BF16 : MOE_DTYPE_F32, &ck);
+    }
+    if (rc) return rc;
+    moe_host::OssMoeConfig& c = m->tr.config;
+    rc = moe_host::moe_config_from_checkpoint(ck, batch_size, &c);
+    if (rc) return rc;
+    const bool tiled = moe_ckpt_is_mxfp4(ck) != 0;
+    if ((rc = alloc_weights(tiled, m))) return rc;
+    moe_host::OssMoeWeights& w = m->tr.weights;
+    const size_t staging_bytes = moe_ckpt_staging_bytes(ck);
+    uint8_t* staging;
+    if ((rc = dev_alloc(&staging, staging_bytes))) return rc;
+    rc = moe_host::moe_upload_weights(ck, c, w, staging, staging_bytes, nullptr);
+    if (!rc) rc = (int)hipDeviceSynchronize();
+    (void)hipFree(staging);
+    moe_ckpt_close(ck);
+    if (rc) return rc;
+
+    return alloc_state(m);
 }
 
 static int read_floats(const char* path, std::vector<float>* out, size_t count) {
@@ -188,6 +211,102 @@ static int run_layers(int argc, char** argv) {
         return 4;
     }
     std::printf("forward() with the reference's seven arguments: same bits; a group of two shards is refused\n");
+    return 0;
+}
+
+// synth <T> <H> <I> <E> <K> <layers> <steps> <warmup> [flags]: a stack of MXFP4 layers filled on the device by the
+// library's synthetic generator (include/moe_synth.h; stream ids of layer l: 2..9 + 16 l for router weight, router
+// bias, gate/up blocks, gate/up bias, down blocks, down bias, gate/up scales, down scales; input rows: id 1; seed 0;
+// unit FFN norm weights), then <warmup> + <steps> calls of forward() on the evolving residual stream.  Prints one
+// JSON line: wall-clock and HIP-event time per forward() call and the checksum (moe_synth_checksum) of the residual
+// stream after the first call, which a caller that builds the same stack can compare with its own.
+static int run_synth(int argc, char** argv) {
+    if (argc < 10) return 2;
+    const int T = std::atoi(argv[2]), H = std::atoi(argv[3]), I = std::atoi(argv[4]), E = std::atoi(argv[5]),
+              K = std::atoi(argv[6]), L = std::atoi(argv[7]), steps = std::atoi(argv[8]), warmup = std::atoi(argv[9]);
+    if (T < 1 || H < 32 || I < 32 || E < 1 || K < 1 || L < 1 || steps < 1 || warmup < 0) return 2;
+    Model m;
+    m.tr.config = moe_host::OssMoeConfig{H, E, K, I, L, 7.0f, T};
+    if (argc > 10) m.tr.flags = (unsigned)std::atoi(argv[10]);
+    CHECK_RC(alloc_weights(true, &m));
+    CHECK_RC(alloc_state(&m));
+    const moe_host::OssMoeWeights& w = m.tr.weights;
+    const unsigned seed = 0;
+    std::vector<float> table(65536);
+    moe_synth_normal_table(table.data());
+    float* table_d;
+    CHECK_RC(dev_alloc(&table_d, table.size()));
+    m.owned.push_back(table_d);
+    CHECK_RC(hipMemcpy(table_d, table.data(), table.size() * sizeof(float), hipMemcpyHostToDevice));
+    std::vector<uint16_t> ones((size_t)L * H, 0x3F80);  // bf16 1.0
+    CHECK_RC(hipMemcpy(const_cast<moe_bf16_t*>(w.rms_ffn_w), ones.data(), ones.size() * 2, hipMemcpyHostToDevice));
+    size_t bb1, sb1, bb2, sb2;
+    moe_mxfp4_tiled_bytes(2 * I, H, &bb1, &sb1);
+    moe_mxfp4_tiled_bytes(H, I, &bb2, &sb2);
+    const long long nb1 = (long long)E * 2 * I * (H / 32), nb2 = (long long)E * H * (I / 32);  // 32-value groups
+    uint8_t *blocks, *scales;
+    CHECK_RC(dev_alloc(&blocks, (size_t)(nb1 > nb2 ? nb1 : nb2) * 16));
+    CHECK_RC(dev_alloc(&scales, (size_t)(nb1 > nb2 ? nb1 : nb2)));
+    for (int l = 0; l < L; ++l) {
+        const unsigned o = 16u * (unsigned)l;
+        const size_t sl = (size_t)l;
+        CHECK_RC(moe_synth_normal_bf16(const_cast<moe_bf16_t*>(w.w_router) + sl * E * H, (long long)E * H, table_d, 0.02f,
+                                       seed, 2 + o, nullptr));
+        CHECK_RC(moe_synth_normal_bf16(const_cast<moe_bf16_t*>(w.b_router) + sl * E, E, table_d, 0.02f, seed, 3 + o, nullptr));
+        CHECK_RC(moe_synth_normal_bf16(const_cast<moe_bf16_t*>(w.b_mlp1) + sl * E * 2 * I, (long long)E * 2 * I, table_d,
+                                       0.02f, seed, 5 + o, nullptr));
+        CHECK_RC(moe_synth_normal_bf16(const_cast<moe_bf16_t*>(w.b_mlp2) + sl * E * H, (long long)E * H, table_d, 0.02f,
+                                       seed, 7 + o, nullptr));
+        CHECK_RC(moe_synth_bytes(blocks, nb1 * 16, seed, 4 + o, nullptr));
+        CHECK_RC(moe_synth_range_bytes(scales, nb1, seed, 8 + o, 119, 9, nullptr));
+        CHECK_RC(moe_mxfp4_repack(blocks, scales, E, 2 * I, H, const_cast<uint8_t*>(w.w_mlp1_blocks) + sl * E * bb1,
+                                  const_cast<uint8_t*>(w.w_mlp1_scales) + sl * E * sb1, nullptr));
+        CHECK_RC(moe_synth_bytes(blocks, nb2 * 16, seed, 6 + o, nullptr));
+        CHECK_RC(moe_synth_range_bytes(scales, nb2, seed, 9 + o, 119, 9, nullptr));
+        CHECK_RC(moe_mxfp4_repack(blocks, scales, E, H, I, const_cast<uint8_t*>(w.w_mlp2_blocks) + sl * E * bb2,
+                                  const_cast<uint8_t*>(w.w_mlp2_scales) + sl * E * sb2, nullptr));
+    }
+    CHECK_RC(hipDeviceSynchronize());
+    (void)hipFree(blocks);
+    (void)hipFree(scales);
+    CHECK_RC(moe_synth_normal_f32(m.tr.state.x, (long long)T * H, table_d, 1.0f, seed, 1, nullptr));
+
+    std::vector<int> tokens(T, 0), pos(T, 0), idx(T);
+    for (int i = 0; i < T; ++i) idx[i] = i;
+    moe_host::OssExpertParallelGroup group;  // one shard: this GPU
+    unsigned long long* sum_d;
+    CHECK_RC(dev_alloc(&sum_d, MOE_SYNTH_CHECKSUM_WORDS));
+    m.owned.push_back(sum_d);
+    unsigned long long first_sum = 0;
+    hipEvent_t e0, e1;
+    CHECK_RC(hipEventCreate(&e0));
+    CHECK_RC(hipEventCreate(&e1));
+    double wall_ms = 0;
+    float event_ms = 0;
+    for (int it = 0; it < warmup + steps; ++it) {
+        if (it == warmup) {
+            CHECK_RC(hipDeviceSynchronize());
+            CHECK_RC(hipEventRecord(e0, nullptr));
+            wall_ms = -now_ms();
+        }
+        if (!moe_host::forward(&m.tr, &group, tokens.data(), pos.data(), T, idx.data(), T)) CHECK_RC(m.tr.last_error);
+        if (it == 0) {
+            if (((size_t)T * H * 4) % 16 == 0) {
+                CHECK_RC(moe_synth_checksum(m.tr.state.x, (long long)T * H * 4, sum_d, nullptr));
+                CHECK_RC(hipMemcpy(&first_sum, sum_d, 8, hipMemcpyDeviceToHost));
+            }
+        }
+    }
+    CHECK_RC(hipEventRecord(e1, nullptr));
+    CHECK_RC(hipDeviceSynchronize());
+    wall_ms += now_ms();
+    CHECK_RC(hipEventElapsedTime(&event_ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    std::printf("{\"mode\": \"synth\", \"T\": %d, \"H\": %d, \"I\": %d, \"E\": %d, \"K\": %d, \"layers\": %d, "
+                "\"steps\": %d, \"warmup\": %d, \"flags\": %u, \"ms_per_forward_wall\": %.6f, "
+                "\"ms_per_forward_events\": %.6f, \"x_checksum_after_first_forward\": %llu}\n",
+                T, H, I, E, K, L, steps, warmup, m.tr.flags, wall_ms / steps, (double)event_ms / steps, first_sum);
     return 0;
 }
 
@@ -366,6 +485,7 @@ int main(int argc, char** argv) {
     if (argc >= 2 && std::string(argv[1]) == "layers") return run_layers(argc, argv);
     if (argc >= 2 && std::string(argv[1]) == "dropin") return run_dropin(argc, argv);
     if (argc >= 2 && std::string(argv[1]) == "getp") return run_getp(argc, argv);
-    std::fprintf(stderr, "usage: %s layers|dropin|getp|requests|verify ... (see the head of moe_stack_main.cpp)\n", argv[0]);
+    if (argc >= 2 && std::string(argv[1]) == "synth") return run_synth(argc, argv);
+    std::fprintf(stderr, "usage: %s layers|dropin|getp|synth|requests|verify ... (see the head of moe_stack_main.cpp)\n", argv[0]);
     return 2;
 }

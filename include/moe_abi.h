@@ -381,6 +381,14 @@ MOE_API int moe_synth_bytes(uint8_t* dst, long long n, unsigned seed, unsigned t
 MOE_API int moe_synth_range_bytes(uint8_t* dst, long long n, unsigned seed, unsigned tensor_id, unsigned lo,
                           unsigned span, moe_stream_t stream);
 
+/* Checksum of a device buffer: out_d[0] = sum of its 32-bit little-endian words modulo 2^64.  n_bytes is a positive
+ * multiple of 16, src is 16-byte aligned, out_d points to MOE_SYNTH_CHECKSUM_WORDS 64-bit words of device memory
+ * (word 0 is the result, the rest per-block partial sums).  The launch only reads src, each byte once, so timed over
+ * a buffer far larger than the caches it measures the read rate the device's memory sustains; the host generator
+ * gives the expected value for a buffer filled by the moe_synth_* entries above.  No counterpart in the reference. */
+#define MOE_SYNTH_CHECKSUM_WORDS 2049
+MOE_API int moe_synth_checksum(const void* src, long long n_bytes, unsigned long long* out_d, moe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,7 @@ def _load():
         "oracle_moe_layer": (_i, [_i, _i, _i, _i, _i, _f] + [_vp] * 12),
         "oracle_mxfp4_to_bf16_bits": (_c.c_uint16, [_u, _u]),
         "oracle_dequant_mxfp4": (None, [_vp, _vp, _ll, _vp]),
+        "oracle_dequant_mxfp4_f32": (None, [_vp, _vp, _ll, _vp]),
         "oracle_bf16_to_f32": (None, [_vp, _ll, _vp]),
         "oracle_f32_to_bf16": (None, [_vp, _ll, _vp]),
         "oracle_bucket": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
@@ -164,9 +165,24 @@ def dequant_mxfp4(blocks, scales):
     return out
 
 
-def bf16_to_f32(bits):
+def dequant_mxfp4_f32(blocks, scales, out=None):
+    """dequant_mxfp4 widened to fp32 in the same pass; `out` (C-contiguous fp32 of the result's size) is filled in
+    place when given."""
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    scales = np.ascontiguousarray(scales, dtype=np.uint8)
+    assert blocks.shape[:-1] == scales.shape and blocks.shape[-1] == 16
+    if out is None:
+        out = np.empty(scales.shape[:-1] + (scales.shape[-1] * 32,), dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous and out.size == scales.size * 32
+    _lib.oracle_dequant_mxfp4_f32(_p(blocks), _p(scales), scales.size, _p(out))
+    return out
+
+
+def bf16_to_f32(bits, out=None):
     bits = np.ascontiguousarray(bits, dtype=np.uint16)
-    out = np.empty(bits.shape, dtype=np.float32)
+    if out is None:
+        out = np.empty(bits.shape, dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous and out.size == bits.size
     _lib.oracle_bf16_to_f32(_p(bits), bits.size, _p(out))
     return out
 

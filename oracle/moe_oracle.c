@@ -313,6 +313,21 @@ ORACLE_API void oracle_dequant_mxfp4(const uint8_t* blocks, const uint8_t* scale
     }
 }
 
+/* The same decoder widened to fp32 in one pass (bf16 -> fp32 is exact): fills the fp32 expert tensors the CPU
+ * path holds without a bf16 copy in between. */
+ORACLE_API void oracle_dequant_mxfp4_f32(const uint8_t* blocks, const uint8_t* scales, long long n_blocks,
+                                         float* out) {
+#pragma omp parallel for
+    for (long long g = 0; g < n_blocks; ++g) {
+        unsigned s = scales[g];
+        for (int b = 0; b < 16; ++b) {
+            unsigned byte = blocks[g * 16 + b];
+            out[g * 32 + 2 * b] = moe_synth_bf16_bits_to_f32(oracle_mxfp4_to_bf16_bits(byte & 0xFu, s));
+            out[g * 32 + 2 * b + 1] = moe_synth_bf16_bits_to_f32(oracle_mxfp4_to_bf16_bits(byte >> 4, s));
+        }
+    }
+}
+
 /* bf16 bits -> fp32 array (how the reference's CPU path holds every weight) */
 ORACLE_API void oracle_bf16_to_f32(const uint16_t* in, long long n, float* out) {
 #pragma omp parallel for

@@ -34,7 +34,7 @@ def host_layer(oracle, wl, shape, layer=0, experts=None):
             per = int(np.prod(d[1:]))
             full = np.zeros(d, dtype=np.float32)
             for e in todo:
-                full[e] = oracle.bf16_to_f32(host_tensor(oracle, d[1:], k, a, shape.seed, start=e * per))
+                oracle.bf16_to_f32(host_tensor(oracle, d[1:], k, a, shape.seed, start=e * per), out=full[e])
         else:
             db, kb, ab = specs[name + "_blocks"]
             ds, ks, as_ = specs[name + "_scales"]
@@ -47,7 +47,7 @@ def host_layer(oracle, wl, shape, layer=0, experts=None):
             for e in todo:
                 blocks = host_tensor(oracle, db[1:], kb, ab, shape.seed, start=e * per_b)
                 scales = host_tensor(oracle, ds[1:], ks, as_, shape.seed, start=e * per_s)
-                full[e] = oracle.bf16_to_f32(oracle.dequant_mxfp4(blocks, scales))
+                oracle.dequant_mxfp4_f32(blocks, scales, out=full[e])
                 if keep:
                     out[name + "_blocks"][e], out[name + "_scales"][e] = blocks, scales
         out[name] = full

@@ -311,3 +311,25 @@ def test_cpp_decode_loop_vs_oracle_loop(oracle, dev, tmp_path):
     print("  decode loop: %d steps, worst rel err of a step %.3e, %d sampled tokens pinned by the oracle, %d too close "
           "to call" % (len(records), worst, decided, undecided), flush=True)
     assert decided > 4 * max(1, undecided)
+
+
+def test_cpp_synthetic_stack_equals_the_python_driven_stack(pkg, wl, dev):
+    """`moe_stack_main synth` builds the synthetic MXFP4 stack the benchmark times (device generator, same stream ids)
+    and runs it through the C++ forward(); the Python-driven DeviceStack over the same tensors must leave the same
+    residual stream bit for bit (compared through moe_synth_checksum, which both sides compute on the device)."""
+    import json
+    import torch
+    shape = wl.MoeShape("synth_small", T=48, H=256, I=128, E=8, K=2, fmt="mxfp4", layers=3)
+    r = run("synth", shape.T, shape.H, shape.I, shape.E, shape.K, shape.layers, 2, 1)
+    assert r.returncode == 0, r.stdout + r.stderr
+    rec = json.loads(r.stdout.strip().splitlines()[-1])
+    assert rec["layers"] == 3 and rec["ms_per_forward_events"] > 0 and rec["ms_per_forward_wall"] > 0
+    table = pkg.normal_table()
+    stack = wl.DeviceStack(shape, table, dev)
+    x = wl.make_device_input(shape, table, dev)
+    stack.prepare(x)
+    stack.forward()
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(x).all()) and float(x.abs().max()) > 0
+    got = int(pkg.synth_checksum(x)[0].item()) & ((1 << 64) - 1)
+    assert got == rec["x_checksum_after_first_forward"]

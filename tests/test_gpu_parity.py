@@ -48,6 +48,30 @@ def test_device_generator_matches_host(pkg, wl, oracle, dev):
     assert np.array_equal(b.cpu().numpy(), oracle.synth_range_bytes((n,), 5, 8, 119, 9))
 
 
+def test_checksum_matches_host_sum(pkg, oracle, dev):
+    """moe_synth_checksum = sum of the buffer's 32-bit words mod 2^64: against numpy on the host generator's bytes
+    (the device buffer is filled by the device generator), from one 16-byte word, over sizes that end inside a
+    thread's chunk, up to more chunks than the launch has blocks; all-ones words so that the 64-bit carry matters;
+    bad sizes and alignments refused."""
+    out = torch.empty(pkg.SYNTH_CHECKSUM_WORDS, dtype=torch.int64, device=dev)
+    for n16 in (1, 255, 256, 1023, 1024, 1025, 5000, 1024 * 2048 + 5, 3 * 1024 * 2048 + 777):
+        n = n16 * 16
+        print("checksum of", n, "bytes", flush=True)
+        b = torch.empty(n, dtype=torch.uint8, device=dev)
+        pkg.synth_bytes(b, 9, 3)
+        got = int(pkg.synth_checksum(b, out=out)[0].item()) & ((1 << 64) - 1)
+        want = int(oracle.synth_bytes((n,), 9, 3).view(np.uint32).sum(dtype=np.uint64))
+        assert got == want, n16
+    ones = torch.full((1 << 20,), -1, dtype=torch.int32, device=dev)  # 2^20 words of 0xFFFFFFFF: sum needs 52 bits
+    assert int(pkg.synth_checksum(ones)[0].item()) == (1 << 20) * 0xFFFFFFFF
+    with pytest.raises(Exception) as e:
+        pkg.synth_checksum(ones.view(torch.uint8)[:24])
+    assert e.value.code == -2  # not a multiple of 16 bytes
+    with pytest.raises(Exception) as e:
+        pkg.synth_checksum(ones.view(torch.uint8)[4:36])
+    assert e.value.code == -6  # source not 16-byte aligned
+
+
 # ---- MXFP4 ---------------------------------------------------------------------------------------
 def test_dequant_exhaustive_bit_exact(pkg, dev):
     """Every (code, scale byte) pair through moe_dequant_mxfp4 against the exact-rational table."""

@@ -201,6 +201,13 @@ def test_dequant_random_matches_table(oracle):
     s = scales[..., None]
     assert np.array_equal(got[..., 0::2], table[lo, s])
     assert np.array_equal(got[..., 1::2], table[hi, s])
+    # the one-pass fp32 form (what fills the CPU path's fp32 expert tensors) is the same values widened; NaN codes
+    # (scale 255) compare as bit patterns
+    wide = oracle.dequant_mxfp4_f32(blocks, scales)
+    assert np.array_equal(wide.view(np.uint32), got.reshape(wide.shape).astype(np.uint32) << 16)
+    into = np.full((3, 5, 90 * 32), 3.0, dtype=np.float32)
+    assert oracle.dequant_mxfp4_f32(blocks, scales, out=into) is into
+    assert np.array_equal(into.view(np.uint32), wide.view(np.uint32))
 
 
 # ---- bucketing: src/hip/scheduler.hip:11-61 ------------------------------------------------------
