@@ -407,23 +407,26 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         // and a half stages) ahead of their use; nothing touches a loaded value before that pair.
         constexpr int DP = 4;
         const int n_pairs = K / 64;
-        const uint8_t* a_ptr[R];
+        // Buffer loads: the expert's matrix is the buffer, the wave-uniform part of an address (row tile, pair,
+        // instruction) is the scalar offset and the lane's part a 32-bit register that never changes, so a load
+        // costs no vector arithmetic (and a read past the matrix would return zeros instead of faulting).
         const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
+        const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(wbase), 0, (int)((uint32_t)a.rows * (uint32_t)K * 2u), 0x00020000);
+        uint32_t a_tile[R];  // wave-uniform byte offset of the row tile's first row
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int row = group * 64 + tile_row_in_group(r0 + r, q & 7);
-            a_ptr[r] = reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 8 * (2 * g + (q >> 3)));
-        }
-        const size_t second_half = (size_t)32 * K * 2;  // tile row q + 8 is weight row + 32 (tile_row_in_group)
+        for (int r = 0; r < R; ++r) a_tile[r] = (uint32_t)(group * 64 + tile_row_in_group(r0 + r, 0)) * (uint32_t)K * 2u;
+        const uint32_t a_lane = (uint32_t)(tile_row_in_group(0, q & 7) * K + 8 * (2 * g + (q >> 3))) * 2u;
+        const uint32_t second_half = 32u * (uint32_t)K * 2u;  // tile row q + 8 is weight row + 32 (tile_row_in_group)
         u32x4 ar[DP][2][R];
         auto load_a = [&](int slot, int pair) {
-            const size_t off = (size_t)(pair < n_pairs ? pair : 0) * 128;  // a padding pair re-reads pair 0 (unused)
+            const uint32_t off = (uint32_t)(pair < n_pairs ? pair : 0) * 128u;  // a padding pair re-reads pair 0 (unused)
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int r = 0; r < R; ++r)
-                    ar[slot][i][r] =
-                        __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a_ptr[r] + off + second_half * i));
+                    ar[slot][i][r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)a_lane,
+                                                                           (int)(a_tile[r] + off + second_half * i), 2 /* nt */);
         };
 #pragma unroll
         for (int i = 0; i < DP - 1; ++i) load_a(i, i);
@@ -1512,7 +1515,11 @@ int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream) {
     if (a.rows % 64 != 0 || a.K % 32 != 0) return MOE_ERR_SHAPE;
     const bool queue = a.work_queue != nullptr;
     if (queue != (epi == EPI_SWIGLU_F32 || epi == EPI_SCATTER)) return MOE_ERR_FORMAT;
-    if (a.format == FMT_BF16) return launch_fmt<FMT_BF16>(a, epi, stream);
+    if (a.format == FMT_BF16) {
+        // the streaming consumers address an expert's matrix through a buffer descriptor: 32-bit byte offsets
+        if ((unsigned long long)a.rows * (unsigned long long)a.K * 2ull > 0x7fffffffull) return MOE_ERR_LIMIT;
+        return launch_fmt<FMT_BF16>(a, epi, stream);
+    }
     if (a.format == FMT_MXFP4) return launch_fmt<FMT_MXFP4>(a, epi, stream);
     return MOE_ERR_FORMAT;
 }
