@@ -106,14 +106,13 @@ def roofline_of(root, shape, res, read_peak):
                  "frac": achieved / MFMA_BF16_PEAK_TFLOPS}, **common)
 
 
-def device_info(torch):
+def device_info(pkg, torch):
     """What the device reports about itself: the peaks above are the part's published ones, not derived from this."""
     pr = torch.cuda.get_device_properties(0)
-    get = lambda name, scale=1: (getattr(pr, name) / scale if hasattr(pr, name) else None)  # noqa: E731
-    return {"name": pr.name, "gcn_arch": getattr(pr, "gcnArchName", None), "compute_units": pr.multi_processor_count,
-            "clock_mhz": get("clock_rate", 1000), "memory_clock_mhz": get("memory_clock_rate", 1000),
-            "memory_bus_bits": get("memory_bus_width"), "l2_bytes": get("L2_cache_size"),
-            "hbm_bytes": pr.total_memory}
+    a = pkg.device_attributes()
+    return {"name": pr.name, "gcn_arch": getattr(pr, "gcnArchName", None), "compute_units": a["compute_units"],
+            "clock_mhz": a["clock_khz"] / 1e3, "memory_clock_mhz": a["memory_clock_khz"] / 1e3,
+            "memory_bus_bits": a["memory_bus_bits"], "l2_bytes": a["l2_bytes"], "hbm_bytes": pr.total_memory}
 
 
 def measure_read_peak(pkg, torch, gib, launches=10):
@@ -416,7 +415,7 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
-    device = device_info(torch)
+    device = device_info(pkg, torch)
     read_peak = measure_read_peak(pkg, torch, args.peak_gib)
     cpu = None if args.no_cpu_baseline else CpuBaseline(ge, wl)
 

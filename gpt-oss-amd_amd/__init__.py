@@ -115,6 +115,7 @@ SIGNATURES = {
     "moe_synth_bytes": (_i, [_vp, _ll, _u, _u, _vp]),
     "moe_synth_range_bytes": (_i, [_vp, _ll, _u, _u, _u, _u, _vp]),
     "moe_synth_checksum": (_i, [_vp, _ll, _vp, _vp]),
+    "moe_device_attributes": (_i, [_vp, _vp, _vp, _vp, _vp]),
 }
 
 
@@ -484,6 +485,13 @@ def synth_normal_bf16(dst, table_d, scale, seed, tensor_id, stream=None):
 
 def synth_bytes(dst, seed, tensor_id, stream=None):
     _check("moe_synth_bytes", _lib.moe_synth_bytes(_ptr(dst), dst.numel(), seed, tensor_id, _stream(stream)))
+
+
+def device_attributes():
+    """dict of what the current device reports: compute_units, clock_khz, memory_clock_khz, memory_bus_bits, l2_bytes."""
+    vals = [_c.c_int(0) for _ in range(5)]
+    _check("moe_device_attributes", _lib.moe_device_attributes(*[ctypes.byref(v) for v in vals]))
+    return dict(zip(("compute_units", "clock_khz", "memory_clock_khz", "memory_bus_bits", "l2_bytes"), [v.value for v in vals]))
 
 
 SYNTH_CHECKSUM_WORDS = 2049

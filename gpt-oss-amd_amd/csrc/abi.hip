@@ -857,6 +857,19 @@ int moe_synth_range_bytes(uint8_t* dst, long long n, unsigned seed, unsigned ten
     return launch_synth(3, dst, n, nullptr, 0.f, seed, tensor_id, lo, span, as_stream(stream));
 }
 
+int moe_device_attributes(int* compute_units, int* clock_khz, int* memory_clock_khz, int* memory_bus_bits,
+                          int* l2_bytes) {
+    int dev = 0;
+    MOE_RETURN_IF_HIP(hipGetDevice(&dev));
+    const struct { int* out; hipDeviceAttribute_t attr; } want[] = {
+        {compute_units, hipDeviceAttributeMultiprocessorCount}, {clock_khz, hipDeviceAttributeClockRate},
+        {memory_clock_khz, hipDeviceAttributeMemoryClockRate}, {memory_bus_bits, hipDeviceAttributeMemoryBusWidth},
+        {l2_bytes, hipDeviceAttributeL2CacheSize}};
+    for (const auto& w : want)
+        if (w.out) MOE_RETURN_IF_HIP(hipDeviceGetAttribute(w.out, w.attr, dev));
+    return MOE_OK;
+}
+
 int moe_synth_checksum(const void* src, long long n_bytes, unsigned long long* out_d, moe_stream_t stream) {
     if (!src || !out_d) return MOE_ERR_NULL;
     if (n_bytes <= 0 || (n_bytes & 15)) return MOE_ERR_SHAPE;

@@ -15,7 +15,9 @@
  *   - returns 0 on success, a negative MOE_ERR_* for a rejected argument, or a positive
  *     hipError_t reported by the runtime.  Nothing exits the process or throws (the reference's
  *     CHECK_HIP prints and calls exit(1): include/model.hpp:8-17);
- *   - re-entrant per device: the library keeps no mutable global state;
+ *   - re-entrant per device: the library keeps no mutable global state, with one exception that
+ *     says so where it is declared (moe_gemm_router_static: a fixed device array per GPU and its
+ *     address, looked up once per device);
  *   - bf16 values cross the boundary as raw 16-bit patterns (moe_bf16_t); the reference's
  *     __hip_bfloat16 has the same size and bit layout.
  */
@@ -78,8 +80,8 @@ MOE_API int moe_gemm_router(float* xout, const float* x_batch, const moe_bf16_t*
 
 /* moe_gemm_router for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference;
- * its argument list is exactly the reference's gemm_router (src/hip/gemms/gemm_router.hip:184-185),
- * so it needs no call-site edit.  The fp64 partial sums live in a fixed device array of
+ * its argument list is moe_gemm_router's without the scratch pair.  The fp64 partial sums live in a
+ * fixed device array of
  * MOE_ROUTER_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
  * ends) instead of a caller buffer; the call allocates nothing.  Same arithmetic and same bits as
  * moe_gemm_router.  Returns MOE_ERR_LIMIT when the partial sums do not fit the array
@@ -388,6 +390,12 @@ MOE_API int moe_synth_range_bytes(uint8_t* dst, long long n, unsigned seed, unsi
  * gives the expected value for a buffer filled by the moe_synth_* entries above.  No counterpart in the reference. */
 #define MOE_SYNTH_CHECKSUM_WORDS 2049
 MOE_API int moe_synth_checksum(const void* src, long long n_bytes, unsigned long long* out_d, moe_stream_t stream);
+
+/* What the current device reports about itself (hipDeviceGetAttribute): compute units, engine clock and memory
+ * clock in kHz, memory bus width in bits, L2 size in bytes.  Any pointer may be NULL.  No counterpart in the
+ * reference; the benchmark prints these beside the published peaks it prices against. */
+MOE_API int moe_device_attributes(int* compute_units, int* clock_khz, int* memory_clock_khz, int* memory_bus_bits,
+                                  int* l2_bytes);
 
 #ifdef __cplusplus
 }
