@@ -486,43 +486,42 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         // on it at load time would pin the wait for the load to the stage that issued it.
         constexpr int D = 4;
         const int G = K / 32;
-        const int rem_groups = G & 3;  // MX blocks in a ragged last stage (0 = none)
-        const size_t tile_bytes = (size_t)G * 256;
-        const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
-        const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
-        const uint8_t* sbase = a.w_scales + (size_t)e * a.s_expert_stride;
-        const uint8_t* wtile[R];  // wave-uniform
-        const uint8_t* stile[R];
+        const uint32_t tile_bytes = (uint32_t)G * 256u;
+        const uint32_t stile_bytes = (uint32_t)ceil_div(ceil_div(G, 4), 4) * 256u;
+        // Buffer loads: the expert's tiled blocks (scales) are the buffer, the wave-uniform part of an address
+        // (row tile, stage) is the scalar offset and the lane's part a constant register.  A read past the
+        // buffer returns zeros instead of faulting, and a read past the tile inside it returns another tile's
+        // bytes: both only ever happen in lanes or stages whose values are dropped (scale 0) or never used,
+        // so no address needs a guard.
+        const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t*>(reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride), 0,
+            (int)a.w_expert_stride, 0x00020000);
+        const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t*>(a.w_scales + (size_t)e * a.s_expert_stride), 0, (int)a.s_expert_stride, 0x00020000);
+        uint32_t wtile[R], stile[R];  // wave-uniform byte offsets inside the expert
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const size_t tile = (size_t)group * 4 + (r0 + r);
-            wtile[r] = wbase + tile * tile_bytes;
-            stile[r] = sbase + tile * stile_bytes;
+            const uint32_t tile = (uint32_t)(group * 4 + (r0 + r));
+            wtile[r] = tile * tile_bytes;
+            stile[r] = tile * stile_bytes;
         }
-        const uint32_t voff_w = (uint32_t)lane * 16;
-        // ragged last stage: a lane group past the last MX block re-reads block 0 and gets scale 0
-        const uint32_t voff_w_ragged = (uint32_t)((g < rem_groups ? lane : q) * 16);
-        const uint32_t voff_s = (uint32_t)lane * 4;
-        const int last_quad = ceil_div(n_stages, 4) - 1;
+        const int voff_w = lane * 16;
+        const int voff_s = lane * 4;
         u32x4 araw[D][R];
         uint32_t sw_cur[R], sw_nxt[R];
-        auto load_a = [&](int slot, int s) {
-            const int su = s < n_stages ? s : 0;  // a padding stage re-reads stage 0 and gets scale 0
-            const bool ragged = rem_groups != 0 && su == n_stages - 1;
-            const uint32_t vo = ragged ? voff_w_ragged : voff_w;
+        auto load_a = [&](int slot, int s) {  // s may lie past the last stage: padding that nobody consumes
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 // non-temporal: a 1 KiB chunk is read once, by this instruction alone, so keeping its
-                // lines in L1/L2 only evicts the activation rows (measured: -5 % kernel time; the bf16
-                // path, where two instructions share each line, and the prefill kernel, where
-                // neighbouring token blocks re-read the weights, are slower with it)
-                araw[slot][r] =
-                    __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wtile[r] + (size_t)su * 1024 + vo));
+                // lines in L1/L2 only evicts the activation rows (measured: -5 % kernel time; the prefill
+                // kernel, where neighbouring token blocks re-read the weights, is slower with it)
+                araw[slot][r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, voff_w, (int)(wtile[r] + (uint32_t)s * 1024u),
+                                                                      2 /* nt */);
         };
         auto load_scales = [&](uint32_t (&dst)[R], int quad) {
-            const size_t off = (size_t)min(quad, last_quad) * 256;
 #pragma unroll
-            for (int r = 0; r < R; ++r) dst[r] = *reinterpret_cast<const uint32_t*>(stile[r] + off + voff_s);
+            for (int r = 0; r < R; ++r)
+                dst[r] = __builtin_amdgcn_raw_buffer_load_b32(s_rsrc, voff_s, (int)(stile[r] + (uint32_t)quad * 256u), 0);
         };
         load_scales(sw_cur, 0);
 #pragma unroll
@@ -534,10 +533,12 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
             constexpr int i = decltype(i_tag)::value;
             load_a((i + D - 1) % D, st + D - 1);
             __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three stages ahead of their use
-            const bool live = !(rem_groups != 0 && st == n_stages - 1 && g >= rem_groups);
+            // In a ragged last stage the lane groups past the last MX block hold another tile's bytes (or zeros);
+            // the tiled scale tensor has scale byte 0 in the slots of blocks that do not exist (moe_mxfp4_repack
+            // clears the tensor before it scatters), which converts to a factor of exactly 0: no select needed.
             float sc[R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu) : 0.0f;
+            for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 u32x4 b[NT];
@@ -723,57 +724,57 @@ MOE_DEVICE void ws_consumer_two(const ExpertGemmArgs& a, const uint8_t* lds, int
         // next pass's unit; those in between are never used and re-read stage 0 with scale 0.
         constexpr int D = 4;
         const int G = K / 32;
-        const int rem_groups = G & 3;  // MX blocks in a ragged last stage (0 = none)
-        const size_t tile_bytes = (size_t)G * 256;
-        const size_t stile_bytes = (size_t)ceil_div(ceil_div(G, 4), 4) * 256;
-        const uint8_t* wbase = reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride;
-        const uint8_t* sbase = a.w_scales + (size_t)e * a.s_expert_stride;
-        const uint8_t* wtile[R];  // wave-uniform
-        const uint8_t* stile[R];
-        const uint8_t* wnext[R];
-        const uint8_t* snext[R];
-        const uint32_t voff_w = (uint32_t)lane * 16;
-        // ragged last stage: a lane group past the last MX block re-reads block 0 and gets scale 0
-        const uint32_t voff_w_ragged = (uint32_t)((g < rem_groups ? lane : q) * 16);
-        const uint32_t voff_s = (uint32_t)lane * 4;
+        const uint32_t tile_bytes = (uint32_t)G * 256u;
+        const uint32_t stile_bytes = (uint32_t)ceil_div(ceil_div(G, 4), 4) * 256u;
+        // Buffer loads: the expert's tiled blocks (scales) are the buffer, the wave-uniform part of an address
+        // (row tile, stage) is the scalar offset and the lane's part a constant register.  A read past the
+        // buffer returns zeros instead of faulting, and a read past the tile inside it returns another tile's
+        // bytes: both only ever happen in lanes or stages whose values are dropped (scale 0) or never used,
+        // so no address needs a guard.
+        const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t*>(reinterpret_cast<const uint8_t*>(a.w) + (size_t)e * a.w_expert_stride), 0,
+            (int)a.w_expert_stride, 0x00020000);
+        const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t*>(a.w_scales + (size_t)e * a.s_expert_stride), 0, (int)a.s_expert_stride, 0x00020000);
+        uint32_t wtile[R], stile[R], wnext[R], snext[R];  // wave-uniform byte offsets inside the expert
+        const int voff_w = lane * 16;
+        const int voff_s = lane * 4;
         const int n_quads = ceil_div(n_stages, 4);
         const int n_pad = 4 * n_quads;
         u32x4 araw[D][R];
         uint32_t sw_cur[R], sw_nxt[R];
+        // stage s of the current pass, or (s >= n_pad) stage s - n_pad of the next pass's unit; a stage number in
+        // between is padding that nobody consumes
         auto load_a = [&](int slot, int s) {
             const bool nxt = TWO && s >= n_pad;  // wave-uniform
-            const int sl = nxt ? s - n_pad : s;
-            const int su = sl < n_stages ? sl : 0;
-            const bool ragged = rem_groups != 0 && su == n_stages - 1;
-            const uint32_t vo = ragged ? voff_w_ragged : voff_w;
+            const uint32_t so = (uint32_t)(nxt ? s - n_pad : s) * 1024u;
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 // non-temporal: a 1 KiB chunk is read once, by this instruction alone, so keeping its
-                // lines in L1/L2 only evicts the activation rows (measured: -5 % kernel time; the bf16
-                // path, where two instructions share each line, and the prefill kernel, where
-                // neighbouring token blocks re-read the weights, are slower with it)
-                araw[slot][r] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4*>((nxt ? wnext[r] : wtile[r]) + (size_t)su * 1024 + vo));
+                // lines in L1/L2 only evicts the activation rows (measured: -5 % kernel time; the prefill
+                // kernel, where neighbouring token blocks re-read the weights, is slower with it)
+                araw[slot][r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, voff_w, (int)((nxt ? wnext[r] : wtile[r]) + so),
+                                                                      2 /* nt */);
         };
         auto load_scales = [&](uint32_t (&dst)[R], int quad) {  // quad n_quads = the next pass's first
             const bool nxt = TWO && quad >= n_quads;
-            const size_t off = (size_t)(nxt ? 0 : min(quad, n_quads - 1)) * 256;
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                dst[r] = *reinterpret_cast<const uint32_t*>((nxt ? snext[r] : stile[r]) + off + voff_s);
+                dst[r] = __builtin_amdgcn_raw_buffer_load_b32(
+                    s_rsrc, voff_s, (int)(nxt ? snext[r] : stile[r] + (uint32_t)quad * 256u), 0);
         };
         // one pass; written out once per pass instead of looped (see the bf16 branch)
         auto do_pass = [&](auto first_tag, int unit, bool more, int gs0) {
             constexpr bool first = decltype(first_tag)::value;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const size_t tile = (size_t)(unit >> 1) * 4 + ((unit & 1) * R + r);
-                const size_t tile_n = more ? (size_t)((unit + unit_step) >> 1) * 4 + (((unit + unit_step) & 1) * R + r) : tile;
-                wtile[r] = wbase + tile * tile_bytes;
-                stile[r] = sbase + tile * stile_bytes;
+                const uint32_t tile = (uint32_t)((unit >> 1) * 4 + ((unit & 1) * R + r));
+                const uint32_t tile_n = more ? (uint32_t)(((unit + unit_step) >> 1) * 4 + (((unit + unit_step) & 1) * R + r)) : tile;
+                wtile[r] = tile * tile_bytes;
+                stile[r] = tile * stile_bytes;
                 if constexpr (TWO) {
-                    wnext[r] = wbase + tile_n * tile_bytes;
-                    snext[r] = sbase + tile_n * stile_bytes;
+                    wnext[r] = tile_n * tile_bytes;
+                    snext[r] = tile_n * stile_bytes;
                 }
             }
             load_bias<R>(a, e, unit >> 1, (unit & 1) * R, bias_raw);  // fetched now, used by the epilogue
@@ -789,14 +790,17 @@ MOE_DEVICE void ws_consumer_two(const ExpertGemmArgs& a, const uint8_t* lds, int
                 __syncthreads();
             }
             // stage st, the i-th of its group of four (i fixes ring slot and scale byte at compile time)
+            // In a ragged last stage the lane groups past the last MX block hold another tile's bytes (or zeros); the
+            // tiled scale tensor has scale byte 0 in the slots of blocks that do not exist (moe_mxfp4_repack clears
+            // the tensor before it scatters), which converts to a factor of exactly 0, so their products vanish
+            // without a select.
             auto stage = [&](auto i_tag, int st) {
                 constexpr int i = decltype(i_tag)::value;
                 load_a((i + D - 1) % D, st + D - 1);
                 __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three stages ahead of their use
-                const bool live = !(rem_groups != 0 && st == n_stages - 1 && g >= rem_groups);
                 float sc[R];
 #pragma unroll
-                for (int r = 0; r < R; ++r) sc[r] = live ? mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu) : 0.0f;
+                for (int r = 0; r < R; ++r) sc[r] = mxfp4_scale_to_f32((sw_cur[r] >> (8 * i)) & 0xFFu);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     u32x4 b[NT];
@@ -1520,7 +1524,10 @@ int launch_expert_stream(const ExpertGemmArgs& a, int epi, hipStream_t stream) {
         if ((unsigned long long)a.rows * (unsigned long long)a.K * 2ull > 0x7fffffffull) return MOE_ERR_LIMIT;
         return launch_fmt<FMT_BF16>(a, epi, stream);
     }
-    if (a.format == FMT_MXFP4) return launch_fmt<FMT_MXFP4>(a, epi, stream);
+    if (a.format == FMT_MXFP4) {
+        if (a.w_expert_stride > 0x7fffffffll || a.s_expert_stride > 0x7fffffffll) return MOE_ERR_LIMIT;
+        return launch_fmt<FMT_MXFP4>(a, epi, stream);
+    }
     return MOE_ERR_FORMAT;
 }
 
