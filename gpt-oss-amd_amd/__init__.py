@@ -325,14 +325,19 @@ def mxfp4_tiled_bytes(rows, K):
     return bb.value, sb.value
 
 
-def mxfp4_repack(blocks, scales, stream=None):
-    """blocks [E, rows, G, 16], scales [E, rows, G] -> (tiled_blocks, tiled_scales) u8 tensors."""
+def mxfp4_repack(blocks, scales, stream=None, out=None):
+    """blocks [E, rows, G, 16], scales [E, rows, G] -> (tiled_blocks, tiled_scales) u8 tensors (`out`: a pair of
+    u8 tensors of E * moe_mxfp4_tiled_bytes to fill instead of new ones)."""
     E, rows, G = scales.shape
     bb, sb = mxfp4_tiled_bytes(rows, G * 32)
     if bb == 0:
         raise MoeError("moe_mxfp4_tiled_bytes", -2)
-    tb = torch.empty(E * bb, dtype=torch.uint8, device=blocks.device)
-    ts = torch.empty(E * sb, dtype=torch.uint8, device=blocks.device)
+    if out is not None:
+        tb, ts = out
+        assert tb.numel() == E * bb and ts.numel() == E * sb and tb.dtype == ts.dtype == torch.uint8
+    else:
+        tb = torch.empty(E * bb, dtype=torch.uint8, device=blocks.device)
+        ts = torch.empty(E * sb, dtype=torch.uint8, device=blocks.device)
     _check("moe_mxfp4_repack", _lib.moe_mxfp4_repack(_ptr(blocks), _ptr(scales), E, rows, G * 32, _ptr(tb), _ptr(ts),
                                                      _stream(stream)))
     return tb, ts

@@ -263,7 +263,12 @@ MOE_API int moe_dequant_mxfp4(const uint8_t* blocks, const uint8_t* scales, long
  *   blocks [E, rows, K/32, 16] u8, scales [E, rows, K/32] u8
  * into the tiled layout the fused kernels stream with 128-bit loads.  K % 32 == 0.
  * moe_mxfp4_tiled_bytes gives the sizes of the two destination buffers for ONE expert; experts
- * are stored back to back.  moe_mxfp4_unpack is the exact inverse. */
+ * are stored back to back.  moe_mxfp4_unpack is the exact inverse.  The tiled scale tensor is
+ * padded to whole groups of four 128-element stages per row tile; moe_mxfp4_repack writes scale
+ * byte 0 into the slots of MX blocks that do not exist (it clears the tensor first), and the
+ * expert kernels rely on that byte: it converts to a factor of exactly 0 for whatever a lane past
+ * the last block of a row has loaded.  A tiled tensor must therefore come from moe_mxfp4_repack
+ * (or moe_ckpt_upload_layer, which calls it). */
 MOE_API void moe_mxfp4_tiled_bytes(int rows, int K, size_t* block_bytes_per_expert,
                            size_t* scale_bytes_per_expert);
 MOE_API int moe_mxfp4_repack(const uint8_t* blocks, const uint8_t* scales, int E, int rows, int K,

@@ -120,6 +120,14 @@ def test_repack_round_trip_and_tiled_dequant(pkg, oracle, dev, E, rows, K):
     want = oracle.dequant_mxfp4(blocks, scales)
     assert np.array_equal(bits_of(pkg.mxfp4_tiled_to_bf16(tb, ts, E, rows, K)), want)
     assert np.array_equal(bits_of(pkg.dequant_mxfp4(db, ds)), want)
+    # The scale slots of MX blocks that do not exist (a ragged last group of four stages) must hold 0 whatever the
+    # destination held before: the expert kernels rely on that byte (a factor of exactly 0) to drop what the lanes past
+    # the last block of a row load.  Every real scale here is non-zero, so the non-zero bytes are exactly the real ones.
+    bb, sb = pkg.mxfp4_tiled_bytes(rows, K)
+    dirty = (torch.full((E * bb,), 0xFF, dtype=torch.uint8, device=dev), torch.full((E * sb,), 0xFF, dtype=torch.uint8, device=dev))
+    tb2, ts2 = pkg.mxfp4_repack(db, ds, out=dirty)
+    assert torch.equal(tb2, tb) and torch.equal(ts2, ts)
+    assert int((ts2 != 0).sum().item()) == E * rows * (K // 32)
 
 
 # ---- router --------------------------------------------------------------------------------------
