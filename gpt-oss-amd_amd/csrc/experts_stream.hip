@@ -605,115 +605,10 @@ MOE_DEVICE void ws_consumer_two(const ExpertGemmArgs& a, const uint8_t* lds, int
     f32x4 acc[R][NT];
     uint2 bias_raw[R];
 
-    if constexpr (FMT == FMT_BF16) {
-        // The contraction range is walked in pairs of MFMA steps (64 elements = one 128-byte
-        // line of a weight row): in a pair, lane group g takes elements 16g .. 16g+7 in the first
-        // step and 16g+8 .. 16g+15 in the second, so a lane's two 16-byte loads are adjacent and
-        // the four lane groups cover the whole line.  Ring of four pairs, loads issued three
-        // pairs (one and a half stages) ahead of their use; nothing touches a loaded value
-        // before the pair that consumes it.  Pair numbers at or past n_pad (the pair count rounded up
-        // to whole ring revolutions) mean the next pass's unit; those in between are never used and
-        // re-read pair 0.
-        constexpr int DP = 4;
-        const int n_pairs = K / 64;
-        const int n_pad = ((n_stages + 1) & ~1) * 2;
-        const uint16_t* wbase = reinterpret_cast<const uint16_t*>(a.w) + (size_t)e * a.w_expert_stride;
-        auto row_ptr = [&](int unit, int r) {
-            const int row = (unit >> 1) * 64 + tile_row_in_group((unit & 1) * R + r, q);
-            return reinterpret_cast<const uint8_t*>(wbase + (size_t)row * K + 16 * g);
-        };
-        const uint8_t* a_ptr[R];
-        const uint8_t* a_nxt[R];
-        u32x4 ar[DP][2][R];
-        auto load_a = [&](int slot, int pair) {
-            if constexpr (TWO) {
-                const bool nxt = pair >= n_pad;  // wave-uniform
-                const int pl = nxt ? pair - n_pad : pair;
-                const size_t off = (size_t)(pl < n_pairs ? pl : 0) * 128;
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int r = 0; r < R; ++r)
-                        ar[slot][h][r] = *reinterpret_cast<const u32x4*>((nxt ? a_nxt[r] : a_ptr[r]) + off + 16 * h);
-            } else {
-                const size_t off = (size_t)(pair < n_pairs ? pair : 0) * 128;  // a padding pair re-reads pair 0 (unused)
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int r = 0; r < R; ++r) ar[slot][h][r] = *reinterpret_cast<const u32x4*>(a_ptr[r] + off + 16 * h);
-            }
-        };
-        // one pass; written out once per pass instead of looped (a loop around the stage code costs the
-        // compiler's register allocation dearly), so a block has at most two passes
-        auto do_pass = [&](auto first_tag, int unit, bool more, int gs0) {
-            constexpr bool first = decltype(first_tag)::value;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                a_ptr[r] = row_ptr(unit, r);
-                if constexpr (TWO) a_nxt[r] = more ? row_ptr(unit + unit_step, r) : a_ptr[r];
-            }
-            load_bias<R>(a, e, unit >> 1, (unit & 1) * R, bias_raw);  // fetched now, used by the epilogue
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int t = 0; t < NT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if constexpr (first) {
-#pragma unroll
-                for (int i = 0; i < DP - 1; ++i) load_a(i, i);
-                if constexpr (PRE) __syncthreads();
-                __syncthreads();
-            }
-            // one stage = two pairs; `ss` (stage parity) fixes the ring slots at compile time
-            auto stage = [&](auto ss_tag, int st) {
-                constexpr int ss = decltype(ss_tag)::value;
-#pragma unroll
-                for (int pp = 0; pp < 2; ++pp) {
-                    constexpr int kSlots = DP;
-                    const int u = 2 * ss + pp;  // ring slot of this pair
-                    const int pair = 2 * st + pp;
-                    load_a((u + kSlots - 1) % kSlots, pair + kSlots - 1);
-                    __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three pairs ahead of their use
-                    const bool live = pair < n_pairs;   // wave-uniform; false only in the second half of a ragged stage
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        u32x4 b[NT];
-#pragma unroll
-                        for (int t = 0; t < NT; ++t) b[t] = b_frag(gs0 + st, 2 * pp + h, t);
-#pragma unroll
-                        for (int r = 0; r < R; ++r) {
-                            const u32x4 av = live ? ar[u][h][r] : u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-                            for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
-                        }
-                    }
-                }
-                __syncthreads();
-            };
-            const int n_even = n_stages & ~1;
-            for (int s0 = 0; s0 < n_even; s0 += 2) {
-                stage(std::integral_constant<int, 0>{}, s0);
-                stage(std::integral_constant<int, 1>{}, s0 + 1);
-            }
-            if (n_stages & 1) {
-                stage(std::integral_constant<int, 0>{}, n_even);
-                if constexpr (TWO) {  // the loads the missing second stage of this ring revolution would have issued
-                    load_a(1, 2 * (n_even + 1) + 3);
-                    load_a(2, 2 * (n_even + 1) + 4);
-                }
-            }
-            stream_epilogue<R, NT, EPI>(a, acc, e, slot_of_row, nrows, unit >> 1, (unit & 1) * R, bias_raw);
-        };
-        if constexpr (TWO) {
-            const int unit1 = unit0 + unit_step;
-            do_pass(std::true_type{}, unit0, passes > 1 && unit1 < unit_end, 0);
-            if (passes > 1) {
-                if (unit1 < unit_end) do_pass(std::false_type{}, unit1, false, n_stages);
-                else for (int i = 0; i < n_stages; ++i) __syncthreads();  // wave-uniform: no unit left for this wave
-            }
-        } else {
-            do_pass(std::true_type{}, unit0, false, 0);
-        }
-    } else {
+    // MXFP4 only: the bf16 stage loops have no registers to spare for a second pass's addresses at 128 registers a
+    // lane (built and measured: 390 spilled registers, gate/up launch 206 against 190 us), so bf16 blocks make one pass.
+    static_assert(FMT == FMT_MXFP4, "two-pass blocks exist for MXFP4 weights only");
+    {
         // Weights: a ring of four stages (one 128-bit load per row tile and stage, issued three
         // stages ahead of its use); scales: one word per row tile covers four stages and is
         // fetched one group of four ahead.  Addresses are a wave-uniform base (scalar registers)
