@@ -307,7 +307,7 @@ def measure_stack(pkg, wl, torch, shape, table, steps, warmup):
     alg_flops = wl.algorithmic_flops(shape) * shape.layers
     work = launch_work(wl, shape, active)
     res = {"workload": shape.name, "ms_per_step": ms, "tokens_per_s": shape.T / (ms * 1e-3), "layers": shape.layers,
-           "steps": steps, "step_ms": stats, "driver": "Python loop over moe_block_forward (workloads.DeviceStack)",
+           "steps": steps, "step_ms": stats, "driver": "one moe_block_forward_layers call per step from Python (workloads.DeviceStack)",
            "stage_ms": dict(zip(pkg.STAGES, [round(v, 5) for v in stage_ms])),
            "block_algorithmic_bytes": alg_bytes,
            "block_hbm_frac": alg_bytes / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9),

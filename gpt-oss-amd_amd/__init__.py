@@ -103,6 +103,7 @@ SIGNATURES = {
     "moe_mxfp4_tiled_to_bf16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "moe_block_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "moe_block_forward": (_i, [_c.POINTER(BlockParams), _vp]),
+    "moe_block_forward_layers": (_i, [_vp, _i, _vp]),
     "moe_block_describe": (_i, [_c.POINTER(BlockParams), _c.c_char_p, _sz]),
     "moe_synth_normal_table": (None, [_vp]),
     "moe_block_down_gemm": (_i, [_c.POINTER(BlockParams), _vp, _vp, _vp]),
@@ -439,6 +440,21 @@ class MoeBlock:
         rc = _lib.moe_block_forward(ctypes.byref(p), stream)
         if rc:
             raise MoeError("moe_block_forward", rc)
+
+
+def pack_layer_params(params):
+    """A ctypes array holding copies of the parameter blocks of consecutive layers, for forward_layers()."""
+    arr = (BlockParams * len(params))()
+    for i, p in enumerate(params):
+        ctypes.memmove(ctypes.byref(arr, i * ctypes.sizeof(BlockParams)), ctypes.byref(p), ctypes.sizeof(BlockParams))
+    return arr
+
+
+def forward_layers(packed, stream, start=0, count=None):
+    """moe_block_forward_layers: layers start .. start+count-1 of a pack_layer_params() array in one call."""
+    n = len(packed) - start if count is None else count
+    _check("moe_block_forward_layers",
+           _lib.moe_block_forward_layers(ctypes.byref(packed, start * ctypes.sizeof(BlockParams)), n, stream))
 
 
 STAGES = ("router_partial", "router_finalize", "bucket", "mlp1_swiglu", "mlp2", "combine")

@@ -694,6 +694,20 @@ static int block_forward_impl(const moe_block_params* caller, moe_stream_t strea
 
 int moe_block_forward(const moe_block_params* p, moe_stream_t stream) { return block_forward_impl(p, stream, nullptr); }
 
+int moe_block_forward_layers(const moe_block_params* params, int n_layers, moe_stream_t stream) {
+    if (!params) return MOE_ERR_NULL;
+    if (n_layers <= 0) return MOE_ERR_SHAPE;
+    const uint8_t* p = reinterpret_cast<const uint8_t*>(params);
+    for (int l = 0; l < n_layers; ++l) {
+        const moe_block_params* q = reinterpret_cast<const moe_block_params*>(p);
+        if (q->struct_bytes < offsetof(moe_block_params, next_norm_weight)) return MOE_ERR_FORMAT;
+        const int rc = block_forward_impl(q, stream, nullptr);
+        if (rc) return rc;
+        p += q->struct_bytes;  // the array's stride is the caller's struct size
+    }
+    return MOE_OK;
+}
+
 int moe_block_describe(const moe_block_params* p, char* text, size_t text_bytes) {
     if (!p || !text) return MOE_ERR_NULL;
     if (text_bytes < 64) return MOE_ERR_LIMIT;

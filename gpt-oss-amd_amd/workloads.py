@@ -192,6 +192,7 @@ class DeviceStack:
                                   next_norm_weight=None if l == last else self.rms_w,
                                   next_norm_out=None if l == last else self.t)
                        for l, blk in enumerate(self.blocks)]
+        self.packed = _pkg.pack_layer_params(self.params)
         self.x = x
 
     def forward(self, stream=None, start=0, stop=None):
@@ -200,8 +201,9 @@ class DeviceStack:
         T, H = self.shape.T, self.shape.H
         stop = len(self.blocks) if stop is None else stop
         _pkg.rmsnorm(self.t, self.x, self.rms_w, T, H, stream=s)  # later layers get theirs from the block before
-        for l in range(start, stop):
-            self.blocks[l].launch(self.params[l], s)
+        # one call issues all the layers: nothing of the host language sits between two layers' launches
+        if stop > start:
+            _pkg.forward_layers(self.packed, s, start, stop - start)
 
 
 # ---- algorithmic work per block (what roofline fractions are computed from) ----------------------

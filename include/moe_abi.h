@@ -341,6 +341,12 @@ MOE_API size_t moe_block_workspace_bytes(int n_tokens, int hidden_dim, int inter
                                  int experts_per_token);
 MOE_API int moe_block_forward(const moe_block_params* params, moe_stream_t stream);
 
+/* moe_block_forward for params[0 .. n_layers-1] in order on one stream: the MoE halves of a layer loop
+ * (src/forward.cpp:258-514 runs one layer after the other the same way) issued by one call, for a host
+ * language whose per-call cost would otherwise sit between the layers.  The array's stride is
+ * params[0].struct_bytes (every element carries the same value).  Stops at the first error. */
+MOE_API int moe_block_forward_layers(const moe_block_params* params, int n_layers, moe_stream_t stream);
+
 /* Which kernels moe_block_forward would launch for these parameters (shapes, format, flags and
  * whether router_score / next_norm_out are set; pointers are not dereferenced and may be NULL), as
  * one line of text: "router=...; bucketing=...; gate_up=<kernel name as a profiler shows it>;
