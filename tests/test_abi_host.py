@@ -75,6 +75,17 @@ def test_entries_reject_bad_arguments_without_a_device(pkg):
     p.struct_bytes = ctypes.sizeof(pkg.BlockParams)
     p.n_tokens, p.hidden_dim, p.intermediate_dim, p.n_experts, p.experts_per_token = 4, 64, 64, 4, 2
     assert L.moe_block_forward(ctypes.byref(p), None) == -1  # NULL tensors
+    # several layers in one call: same checks per element, the array is walked by the caller's struct size
+    assert L.moe_block_forward_layers(None, 2, None) == -1
+    assert L.moe_block_forward_layers(ctypes.byref(p), 0, None) == -2
+    two = pkg.pack_layer_params([p, p])
+    assert ctypes.sizeof(two) == 2 * ctypes.sizeof(pkg.BlockParams)
+    assert L.moe_block_forward_layers(ctypes.byref(two), 2, None) == -1  # NULL tensors in the first element
+    two[0].struct_bytes = 8
+    assert L.moe_block_forward_layers(ctypes.byref(two), 2, None) == -5
+    assert L.moe_synth_checksum(None, 16, None, None) == -1
+    assert L.moe_synth_checksum(16, 24, 16, None) == -2     # not a multiple of 16 bytes
+    assert L.moe_synth_checksum(8, 32, 16, None) == -6      # source not 16-byte aligned
     with pytest.raises(pkg.MoeError):
         pkg._check("x", -2)
 

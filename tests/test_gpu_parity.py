@@ -72,6 +72,14 @@ def test_checksum_matches_host_sum(pkg, oracle, dev):
     assert e.value.code == -6  # source not 16-byte aligned
 
 
+def test_device_attributes_are_those_of_the_part(pkg, dev):
+    a = pkg.device_attributes()
+    pr = torch.cuda.get_device_properties(0)
+    assert a["compute_units"] == pr.multi_processor_count and a["compute_units"] >= 64
+    assert 500_000 <= a["clock_khz"] <= 4_000_000 and a["memory_clock_khz"] > 0
+    assert a["memory_bus_bits"] >= 1024 and a["l2_bytes"] >= 1 << 20
+
+
 # ---- MXFP4 ---------------------------------------------------------------------------------------
 def test_dequant_exhaustive_bit_exact(pkg, dev):
     """Every (code, scale byte) pair through moe_dequant_mxfp4 against the exact-rational table."""
