@@ -11,8 +11,9 @@ peak (2.5 PFLOP/s bf16 MFMA peak).  `roofline.practical_peak` is measured in the
 streaming read of 4 GiB through the library's checksum kernel (every byte fetched once, nothing
 written), so the gap between a kernel and what this device's memory sustains can be read off beside
 the gap to the nominal figure.  `device` holds the CU count and the clocks the device reports.
-`ms_per_step` is the wall-clock mean over the timed steps; `step_ms` adds the median and the minimum
-of per-step HIP-event times.  Every workload under `also` carries the same objects for its own
+`ms_per_step` is the wall-clock mean over the timed steps (preceded by max(--warmup, 100) untimed ones:
+the device's step time needs about 40 steps to settle after a change of workload); `step_ms` adds the
+median and the minimum of per-step HIP-event times.  Every workload under `also` carries the same objects for its own
 launches; the MXFP4 decode workload also runs with three copies of its expert tensors used in turn
 (1.3 GB, five times the 256 MB Infinity Cache) next to the single-copy figure, and the 36-layer stack
 is also timed through the C++ forward() of host/moe_forward.hpp (host/bin/moe_stack_main synth, a child
