@@ -795,11 +795,17 @@ MOE_DEVICE void ws_block_coords(const ExpertGemmArgs& a, int& item, int& rb) {
     rb = a.xcd_tiles ? (blockIdx.x >> 3) % n_rb : blockIdx.x % n_rb;
 }
 
-// the row units of the weight matrix are spread evenly over the row blocks: block rb takes [u0, u1)
+// the row units of the weight matrix are spread evenly over the row blocks (sizes differ by at most one unit):
+// block rb takes [u0, u1)
 MOE_DEVICE void ws_row_units(const ExpertGemmArgs& a, int rb, int& u0, int& u1) {
     const int units = a.rows / 32;
-    u0 = (int)((long long)rb * units / a.row_blocks);
-    u1 = (int)((long long)(rb + 1) * units / a.row_blocks);
+    // the blocks with one unit more come first in the launch order: when the blocks take more than one round
+    // over the compute units, the second-round blocks are handed out in that order to the units as they finish,
+    // so a unit whose first block was a long one ends with a short one (measured: bf16 gate/up launch at 256
+    // tokens, 512 blocks of 11 or 12 units, -3 %)
+    const int q = units / a.row_blocks, rem = units - q * a.row_blocks;
+    u0 = rb * q + min(rb, rem);
+    u1 = u0 + q + (rb < rem ? 1 : 0);
 }
 
 // Token blocks from the tile map written by the bucketing kernel.
