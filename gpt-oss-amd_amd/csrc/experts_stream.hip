@@ -366,10 +366,12 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row
 // first weight loads have been issued (the kernel that finds the bucket itself completes the bucket
 // list behind that barrier; the consumers need the list only in their epilogue, so their weights are
 // already on the way while the producers read it).
-template <int FMT, int NT, int EPI, bool PRE = false, class SlotFn>
-MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows, int unit,
+// tile0: the first of the wave's R row tiles of 16 weight rows (R = 2: a row unit, tile0 even; R = 1: a single
+// tile, for blocks whose range of tiles starts or ends inside a unit).
+template <int FMT, int NT, int EPI, bool PRE = false, int R = 2, class SlotFn>
+MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows, int tile0,
                             bool active) {
-    constexpr int R = 2;
+    static_assert(R == 1 || R == 2, "one or two row tiles per wave");
     const int lane = threadIdx.x & 63;
     const int g = lane >> 4;
     const int q = lane & 15;
@@ -379,8 +381,8 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
         for (int i = 0; i <= n_stages + (PRE ? 1 : 0); ++i) __syncthreads();
         return;
     }
-    const int group = unit >> 1;
-    const int r0 = (unit & 1) * R;
+    const int group = tile0 >> 2;
+    const int r0 = tile0 & 3;
     uint2 bias_raw[R];  // fetched now, used by the epilogue
     load_bias<R>(a, e, group, r0, bias_raw);
     const uint8_t* const lds_rd = lds + (size_t)q * 256;
@@ -761,12 +763,31 @@ template <int FMT, int NT, int EPI, bool PRE, bool TWO, class SlotFn>
 MOE_DEVICE void ws_consume_units(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows,
                                  int unit0, int unit_end, int unit_step, int passes) {
     if constexpr (TWO) ws_consumer_two<FMT, NT, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit0, unit_end, unit_step, passes);
-    else ws_consumer<FMT, NT, EPI, PRE>(a, lds, e, slot_of_row, nrows, unit0, unit0 < unit_end);
+    else ws_consumer<FMT, NT, EPI, PRE>(a, lds, e, slot_of_row, nrows, 2 * unit0, unit0 < unit_end);
+}
+
+// The same for a block whose rows are a range of row TILES [t0, t1) that need not start or end on a unit: a
+// tile in front of the first whole unit goes to wave 0 and one behind the last whole unit to the wave after the
+// last whole unit, each as a single tile; the launch sees to it that CONS waves are enough.
+template <int FMT, int NT, int EPI, bool PRE, class SlotFn>
+MOE_DEVICE void ws_consume_tiles(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows,
+                                 int t0, int t1, int wave) {
+    const int lead = t0 & 1;
+    const int first = (wave == 0 || !lead) ? t0 + 2 * wave : t0 + 2 * wave - 1;  // wave-uniform
+    if (lead && wave == 0) {
+        ws_consumer<FMT, NT, EPI, PRE, 1>(a, lds, e, slot_of_row, nrows, t0, true);
+    } else if (first + 1 == t1) {
+        ws_consumer<FMT, NT, EPI, PRE, 1>(a, lds, e, slot_of_row, nrows, first, true);
+    } else {
+        ws_consumer<FMT, NT, EPI, PRE, 2>(a, lds, e, slot_of_row, nrows, first, first + 1 < t1);
+    }
 }
 
 // One token block: the producer or consumer role of this wave, for the block's token-tile count.
-// u0, u1: the block's row units [u0, u1), walked in passes of CONS units.
-template <int FMT, int EPI, int CONS, int PROD, bool PRE = false, bool TWO = false, class RowFn, class SlotFn>
+// u0, u1: the block's row units [u0, u1), walked in passes of CONS units; with TILES its row tiles [u0, u1)
+// (one pass, see ws_consume_tiles).
+template <int FMT, int EPI, int CONS, int PROD, bool PRE = false, bool TWO = false, bool TILES = false, class RowFn,
+          class SlotFn>
 MOE_DEVICE void ws_token_block(const ExpertGemmArgs& a, uint8_t* lds, int wave, int u0, int u1, int e, RowFn act_row,
                                SlotFn slot_of_row, int nrows) {
     const int nt = (nrows + 15) >> 4;  // block-uniform
@@ -778,6 +799,12 @@ MOE_DEVICE void ws_token_block(const ExpertGemmArgs& a, uint8_t* lds, int wave, 
         else if (nt == 3) ws_producer<FMT, 3, PROD>(a, lds, act_row, nrows, p, passes);
         else if (nt == 2) ws_producer<FMT, 2, PROD>(a, lds, act_row, nrows, p, passes);
         else ws_producer<FMT, 1, PROD>(a, lds, act_row, nrows, p, passes);
+    } else if constexpr (TILES) {
+        static_assert(!TWO, "a range of tiles is walked in one pass");
+        if (nt == 4) ws_consume_tiles<FMT, 4, EPI, PRE>(a, lds, e, slot_of_row, nrows, u0, u1, wave);
+        else if (nt == 3) ws_consume_tiles<FMT, 3, EPI, PRE>(a, lds, e, slot_of_row, nrows, u0, u1, wave);
+        else if (nt == 2) ws_consume_tiles<FMT, 2, EPI, PRE>(a, lds, e, slot_of_row, nrows, u0, u1, wave);
+        else ws_consume_tiles<FMT, 1, EPI, PRE>(a, lds, e, slot_of_row, nrows, u0, u1, wave);
     } else {
         if (nt == 4) ws_consume_units<FMT, 4, EPI, PRE, TWO>(a, lds, e, slot_of_row, nrows, u0 + wave, u1, CONS, passes);
         else if (nt == 3) ws_consume_units<FMT, 3, EPI, PRE, TWO>(a, lds, e, slot_of_row, nrows, u0 + wave, u1, CONS, passes);
@@ -806,6 +833,23 @@ MOE_DEVICE void ws_row_units(const ExpertGemmArgs& a, int rb, int& u0, int& u1) 
     const int q = units / a.row_blocks, rem = units - q * a.row_blocks;
     u0 = rb * q + min(rb, rem);
     u1 = u0 + q + (rb < rem ? 1 : 0);
+}
+
+// The same split in row tiles of 16 rows (two per unit), for blocks that make one pass: block sizes then differ
+// by half a unit at most.  A block whose range starts or ends inside a unit needs a wave for each of those single
+// tiles, so this split is only used while a block stays below 2 CONS tiles; otherwise the unit split, in tiles.
+template <int CONS>
+MOE_DEVICE void ws_row_tiles(const ExpertGemmArgs& a, int rb, int& t0, int& t1) {
+    const int tiles = a.rows / 16;
+    const int q = tiles / a.row_blocks, rem = tiles - q * a.row_blocks;
+    if (q + (rem ? 1 : 0) <= 2 * CONS - 1) {
+        t0 = rb * q + min(rb, rem);
+        t1 = t0 + q + (rb < rem ? 1 : 0);
+    } else {
+        ws_row_units(a, rb, t0, t1);
+        t0 *= 2;
+        t1 *= 2;
+    }
 }
 
 // Token blocks from the tile map written by the bucketing kernel.
@@ -857,8 +901,12 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_chunks = (a.n_assign + 63) >> 6;
+    // bf16 blocks make one pass over their rows and take them as a range of row tiles; MXFP4 blocks make up to two
+    // passes of CONS units each, whose time does not depend on how many units a pass holds
+    constexpr bool TILES = !TWO && FMT == FMT_BF16;
     int u0, u1;
-    ws_row_units(a, rb, u0, u1);
+    if constexpr (TILES) ws_row_tiles<CONS>(a, rb, u0, u1);
+    else ws_row_units(a, rb, u0, u1);
     int n_bucket;
     {
         // this wave's chunks of the assignment list
@@ -901,7 +949,7 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
     // code; what is left are whole blocks of 64 rows, run by a loop that holds the four-tile variant
     // only (a loop around all tile-count variants costs every variant 30 registers per lane).
     const int first = n_bucket - ((n_bucket - 1) & ~63);
-    ws_token_block<FMT, EPI, CONS, PROD, true, TWO>(
+    ws_token_block<FMT, EPI, CONS, PROD, true, TWO, TILES>(
         a, lds, wave, u0, u1, e, [&](int i) { return a.gather ? token_of(bucket[i]) : bucket[i]; },
         [&](int i) { return bucket[i]; }, first);
     const int passes = TWO ? min(2, max(1, ceil_div(u1 - u0, CONS))) : 1;
@@ -909,6 +957,7 @@ __global__ __launch_bounds__((CONS + PROD) * 64, (CONS + PROD > 12) ? 4 : 3) voi
         auto act_row = [&](int i) { return a.gather ? token_of(bucket[row0 + i]) : bucket[row0 + i]; };
         auto slot_of_row = [&](int i) { return bucket[row0 + i]; };
         if (wave >= CONS) ws_producer<FMT, 4, PROD>(a, lds, act_row, 64, wave - CONS, passes);
+        else if constexpr (TILES) ws_consume_tiles<FMT, 4, EPI, false>(a, lds, e, slot_of_row, 64, u0, u1, wave);
         else ws_consume_units<FMT, 4, EPI, false, TWO>(a, lds, e, slot_of_row, 64, u0 + wave, u1, CONS, passes);
     }
 }

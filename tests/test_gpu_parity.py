@@ -269,6 +269,8 @@ SMALL = [
     (700, 192, 64, 64, 8, "bf16"),
     (400, 576, 448, 8, 2, "bf16"),
     (97, 576, 832, 2, 2, "bf16"),
+    # 56 and 52 row tiles over three row blocks (19, 19, 18 and 18, 17, 17): bf16 blocks that start or end inside a row unit
+    (40, 832, 448, 4, 2, "bf16"),
 ]
 
 
