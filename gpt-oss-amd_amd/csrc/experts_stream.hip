@@ -772,7 +772,7 @@ MOE_DEVICE void ws_consume_units(const ExpertGemmArgs& a, const uint8_t* lds, in
 template <int FMT, int NT, int EPI, bool PRE, class SlotFn>
 MOE_DEVICE void ws_consume_tiles(const ExpertGemmArgs& a, const uint8_t* lds, int e, SlotFn slot_of_row, int nrows,
                                  int t0, int t1, int wave) {
-    const int lead = t0 & 1;
+    const int lead = (t0 & 1) && t0 < t1;  // an empty range has no waves at work
     const int first = (wave == 0 || !lead) ? t0 + 2 * wave : t0 + 2 * wave - 1;  // wave-uniform
     if (lead && wave == 0) {
         ws_consumer<FMT, NT, EPI, PRE, 1>(a, lds, e, slot_of_row, nrows, t0, true);
