@@ -304,23 +304,36 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row
     const int K = a.K;
     const int n_stages = ceil_div(K, kStageElems);
     // this wave moves row blocks BP*p .. BP*p + BP-1 of every token tile; in the bucket's last token
-    // tile only those that hold a row of the bucket (n_last of them, the others stay stale in LDS:
-    // the accumulator columns they feed are never stored)
+    // tile only those that hold a row of the bucket (n_last of them), and of those only the lanes whose row
+    // exists.  The places of the rows past the bucket's end are cleared once, below, in every ring slot, and no
+    // load ever writes them.  The accumulator columns they feed are never stored, so any value would do for
+    // the result; zeros are what the matrix pipe spends least on (measured on a synthetic kernel of this shape:
+    // a token tile of zeros costs a stage 0.0-0.1 us, a tile of arbitrary values 0.15-0.25 us, at the same
+    // instruction count), and a bucket of 33 rows has 15 such columns in its third tile.
     int n_last = 0;
 #pragma unroll
     for (int ii = 0; ii < BP; ++ii) n_last += (16 * (NT - 1) + 4 * (BP * p + ii) < nrows) ? 1 : 0;
     const uint8_t* row[NT][BP];
     int chunk[BP];
+    bool last_live[BP];  // this lane's row of the last token tile exists
 #pragma unroll
     for (int ii = 0; ii < BP; ++ii) {
         const int q = 4 * (BP * p + ii) + sub;
         chunk[ii] = ws_chunk_at<FMT>(pos ^ q);
+        last_live[ii] = 16 * (NT - 1) + q < nrows;
+        if (!last_live[ii]) {
+#pragma unroll
+            for (int slot = 0; slot < kWsRing; ++slot)
+                *reinterpret_cast<u32x4*>(lds + (size_t)slot * kLdsStageBytes + (NT - 1) * 4096 + (BP * p + ii) * 1024 +
+                                          lane * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int idx = min(t * 16 + q, nrows - 1);
             row[t][ii] = reinterpret_cast<const uint8_t*>(a.act + (size_t)act_row(idx) * K);
         }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the clearing stores, before this wave's first barrier
     // stage st of the rows into ring slot gs % 4 (gs counts stages over all passes)
     auto issue = [&](int gs, int st) {
         uint8_t* slot = lds + (size_t)(gs & (kWsRing - 1)) * kLdsStageBytes;
@@ -329,8 +342,10 @@ MOE_DEVICE void ws_producer(const ExpertGemmArgs& a, uint8_t* lds, RowFn act_row
             const int k = st * kStageElems + 8 * chunk[ii];
             const size_t off = (k < K) ? (size_t)k * 2 : 0;  // a position past the row re-reads its start
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-                if (t < NT - 1 || ii < n_last) dma16(row[t][ii] + off, slot + t * 4096 + (BP * p + ii) * 1024);
+            for (int t = 0; t < NT - 1; ++t) dma16(row[t][ii] + off, slot + t * 4096 + (BP * p + ii) * 1024);
+            // the last tile: a block without a row is skipped (wave-uniform, the waits below count on it); in a block
+            // with rows the lanes without one sit the instruction out (it is issued, and counted, all the same)
+            if (ii < n_last && last_live[ii]) dma16(row[NT - 1][ii] + off, slot + (NT - 1) * 4096 + (BP * p + ii) * 1024);
         }
     };
     // stage s has landed once only the loads of the two stages issued after it are outstanding
