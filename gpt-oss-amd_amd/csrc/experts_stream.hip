@@ -463,20 +463,33 @@ MOE_DEVICE void ws_consumer(const ExpertGemmArgs& a, const uint8_t* lds, int e, 
                 __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, three pairs ahead of their use
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    u32x4 b[NT];
+                    u32x4 av[R];
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) b[t] = b_frag(st, 2 * pp + h, t);
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        u32x4 av;
+                    for (int r = 0; r < R; ++r)
 #pragma unroll
                         for (int d = 0; d < 4; ++d)
-                            av[d] = h == 0 ? (uint32_t)__builtin_amdgcn_update_dpp((int)ar[u][0][r][d], (int)ar[u][1][r][d],
-                                                                                   0x128, 0xF, 0xC, false)
-                                           : (uint32_t)__builtin_amdgcn_update_dpp((int)ar[u][1][r][d], (int)ar[u][0][r][d],
-                                                                                   0x128, 0xF, 0x3, false);
+                            av[r][d] = h == 0 ? (uint32_t)__builtin_amdgcn_update_dpp((int)ar[u][0][r][d], (int)ar[u][1][r][d],
+                                                                                      0x128, 0xF, 0xC, false)
+                                              : (uint32_t)__builtin_amdgcn_update_dpp((int)ar[u][1][r][d], (int)ar[u][0][r][d],
+                                                                                      0x128, 0xF, 0x3, false);
+                    if constexpr (NT == 4) {
+                        // four token tiles: one activation operand at a time, for both row tiles (the four of them
+                        // held at once cost the registers that keep this loop free of spills; a spill access in
+                        // here waits for every weight load in flight, since it counts in the same counter)
 #pragma unroll
-                        for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av, b[t], acc[r][t]);
+                        for (int t = 0; t < NT; ++t) {
+                            const u32x4 b = b_frag(st, 2 * pp + h, t);
+#pragma unroll
+                            for (int r = 0; r < R; ++r) acc[r][t] = mfma_16x16x32(av[r], b, acc[r][t]);
+                        }
+                    } else {
+                        u32x4 b[NT];
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) b[t] = b_frag(st, 2 * pp + h, t);
+#pragma unroll
+                        for (int r = 0; r < R; ++r)
+#pragma unroll
+                            for (int t = 0; t < NT; ++t) acc[r][t] = mfma_16x16x32(av[r], b[t], acc[r][t]);
                     }
                 }
             }
